@@ -97,7 +97,7 @@ class LLMEngine:
                                    ahead_over_block_edges=(cfg.decode_prelaunch_edges and os.environ.get(
                                        "MINIVLLM_NO_EDGE_PRELAUNCH") != "1"),
                                    num_state_slots=self.model_runner.num_state_slots,
-                                   prefix_caching=not self.model_runner.num_state_slots)
+                                   prefix_caching=self.model_runner.prefix_cacheable)
         self._given: Dict[str, Sequence] = {}
         self.tokenizer = load_tokenizer(cfg.model_name_or_path, cfg.model.vocab_size)
         self.stats = EngineStats()

@@ -179,6 +179,10 @@ class ModelRunner:
         self.hybrid = hasattr(self.model, "state_layers")
         self.needs_aux_rows = bool(getattr(self.model, "needs_aux_rows", False))
         self.num_state_slots = cfg.max_num_sequences if self.hybrid and self.model.state_layers() else 0
+        # a cached KV block says nothing about recurrent state; a family may also opt out
+        # because its layers keep several caches per block id (``prefix_cacheable = False``)
+        self.prefix_cacheable = bool(not self.num_state_slots
+                                     and getattr(self.model, "prefix_cacheable", True))
         fold = cfg.fold_norm_weights
         if fold is None:
             fold = self.tp == 1 and not pg.collectives_active()

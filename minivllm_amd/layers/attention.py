@@ -216,3 +216,45 @@ class SinkAttention(nn.Module):
                                           None if gate is None else gate[:Bd], out[:Bd],
                                           ctx.max_context_len or None, **opt)
         return out.view(T, self.num_heads * self.v_head_dim)
+
+
+class LatentAttention(nn.Module):
+    """Attention whose keys and values are expansions of one cached latent per token: key of
+    head h = [W_uk_h c | r], value = W_uv_h c, with c the RMS-normed latent (R numbers) and r one
+    rotated key part (P numbers) shared by all heads.  Only c and r are cached, and the
+    expansions are never formed: with a_h = W_uk_h^T q_h the score is (a_h . c + q_rot_h . r) *
+    scale, and the weighted sum of values is W_uv_h applied to the weighted sum of latents.  So
+    this is attention with ONE key/value head whose key row is [c | r] (R + P) and whose value row
+    is c (R), run by ``SinkAttention`` (no sink; its window and kernels), between two batched
+    products per head.  ``up_k`` [H, D, R] and ``up_v`` [H, E, R] are the per-head expansion
+    matrices; ``rotation``: a ``HalfRotation`` over the first entries of the P-part."""
+
+    def __init__(self, num_heads: int, head_dim: int, rot_dim: int, v_head_dim: int, kv_rank: int,
+                 scale: float, window: int, rotation, eps: float):
+        super().__init__()
+        H, D, P, E, R = num_heads, head_dim, rot_dim, v_head_dim, kv_rank
+        self.num_heads, self.head_dim, self.rot_dim, self.v_head_dim, self.kv_rank = H, D, P, E, R
+        self.eps, self.rotation = eps, rotation
+        if rotation.rotary_dim > P:
+            raise ValueError("the rotation covers more entries than the rotated part has")
+        self.core = SinkAttention(H, 1, R + P, R, scale, sink=False, window=window)
+        self.latent_norm = nn.Parameter(torch.ones(R, dtype=torch.float32), requires_grad=False)
+        self.up_k = nn.Parameter(torch.zeros(H, D, R), requires_grad=False)
+        self.up_v = nn.Parameter(torch.zeros(H, E, R), requires_grad=False)
+
+    def forward(self, q: torch.Tensor, dkv: torch.Tensor, core: Optional[SinkAttention] = None
+                ) -> torch.Tensor:
+        """q [T, H, D + P] (the rotated part last), dkv [T, R + P] raw -> [T, H, E] as a
+        transposed view of [H, T, E].  ``core``: the cache holder of this pass (default: the
+        module's own)."""
+        ctx = get_context()
+        core = core or self.core
+        T = q.shape[0]
+        H, D, R = self.num_heads, self.head_dim, self.kv_rank
+        q_abs = torch.bmm(q[:, :, :D].transpose(0, 1), self.up_k)                    # [H, T, R]
+        rot = self.rotation
+        qf = ops.latent_rope_store(q_abs, q, dkv, self.latent_norm, self.eps, ctx.positions,
+                                   rot.inv_freq, rot.rotary_dim, core.k_cache, core.v_cache,
+                                   ctx.slot_mapping)
+        o = core(qf, None).view(T, H, R)
+        return torch.bmm(o.transpose(0, 1), self.up_v.transpose(1, 2)).transpose(0, 1)   # [T, H, E]

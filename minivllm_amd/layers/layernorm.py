@@ -78,3 +78,26 @@ class GroupRMSNorm(nn.Module):
 
     def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         return ops.group_rms_norm(x, self.weight, self.groups, self.eps, out_dtype or x.dtype)
+
+
+class ScalarRMSNorm(nn.Module):
+    """RMS norm whose gain is ONE number for all coordinates: ``x / rms(x) * gain`` (eps inside
+    the root).  The gain is kept as a host float besides the parameter, so that the fused form
+    (``ops.residual_sum_norm``: update of the fp32 stream + this norm) takes it as a kernel
+    argument.  Applied alone it normalises the rows it is given."""
+
+    def __init__(self, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones((), dtype=torch.float32), requires_grad=False)
+        self.gain = 1.0
+
+    @torch.no_grad()
+    def load(self, t: torch.Tensor) -> None:
+        if t.numel() != 1:
+            raise ValueError(f"a scalar norm takes one number, got shape {tuple(t.shape)}")
+        self.weight.copy_(t.reshape(()).to(torch.float32))
+        self.gain = float(t.reshape(()).float())
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return ops.residual_sum_norm(x, (), (), self.gain, self.eps, out_dtype or x.dtype)

@@ -63,3 +63,21 @@ class PairRotaryEmbedding(nn.Module):
         self.register_buffer("cos_sin_cache",
                              torch_seqmix.pair_cos_sin_table(rotary_dim, max_position, base, scaling),
                              persistent=False)
+
+
+class HalfRotation(nn.Module):
+    """Rotation in the half-split layout on the first ``rotary_dim`` entries of a vector: entry i
+    is paired with entry i + rotary_dim/2 and the pair (u, v) at position p becomes
+    (u cos a - v sin a, v cos a + u sin a), a = p * base^(-2i / rotary_dim); later entries pass
+    unchanged.  Owns only the fp32 frequencies (rounded from float64); the angle is the fp32
+    product of position and frequency, formed where the rotation is applied
+    (``ops.latent_rope_store``), so no table and no maximal position."""
+
+    def __init__(self, rotary_dim: int, base: float):
+        super().__init__()
+        if rotary_dim % 2:
+            raise ValueError("rotary_dim must be even")
+        self.rotary_dim, self.base = int(rotary_dim), float(base)
+        i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+        self.register_buffer("inv_freq", (self.base ** (-2.0 * i / max(rotary_dim, 1))).float(),
+                             persistent=False)

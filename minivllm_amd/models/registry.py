@@ -94,3 +94,13 @@ def _ensure_builtin() -> None:
         return PelenexForCausalLM
 
     register(["pelenex"], pelenex_cfg, pelenex_class)
+
+    def kidupel_cfg(c, name):
+        from minivllm_amd.models.kidupel import KidupelConfig
+        return KidupelConfig.from_dict(c, name)
+
+    def kidupel_class():
+        from minivllm_amd.models.kidupel import KidupelForCausalLM
+        return KidupelForCausalLM
+
+    register(["kidupel"], kidupel_cfg, kidupel_class)

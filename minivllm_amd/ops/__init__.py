@@ -306,18 +306,21 @@ def unit_norm_store(q, k, eps, k_cache, v_cache, slot_mapping):
 
 
 def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots,
-                  row_seq=None):
+                  row_seq=None, conv_bias=None, ssd=False):
     """``row_seq`` [T] (GPU, prefill-form steps): the sequence of each row, -1 for rows that
-    belong to none; the CPU form walks ``cu_q`` instead."""
+    belong to none; the CPU form walks ``cu_q`` instead.  ``conv_bias`` [C] fp32: added to the
+    convolution before its silu.  ``ssd``: the state-space form (q / k stay as convolved, beta is
+    the step size softplus(a + dt_bias), ``b`` is not read), see ``torch_seqmix.delta_prepare``."""
     if _on_gpu(q):
         return _hybrid().delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state,
-                                       cu_q, positions, slots, row_seq)
+                                       cu_q, positions, slots, row_seq, conv_bias, ssd)
     return torch_seqmix.delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state,
-                                      cu_q, positions, slots)
+                                      cu_q, positions, slots, conv_bias, ssd)
 
 
-def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
-    return _seqmix(qn).delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots)
+def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots, correct=True):
+    """``correct`` False: the update is beta k v^T without the delta rule's correction term."""
+    return _seqmix(qn).delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots, correct)
 
 
 def gated_head_norm(o, w, gate, eps, out_dtype, act="silu"):
@@ -364,3 +367,34 @@ def gla_scan(q, k, v, a_raw, a_bias, tau, state, cu_q, positions, slots):
 
 def gelu_route_scale(up, dense, ff, out_dtype):
     return _seqmix(up).gelu_route_scale(up, dense, ff, out_dtype)
+
+
+# ---- scaled parallel branches, whole-projection norms, attention over a shared latent, xIELU
+def rms_norm_rows(x, w, eps, out_dtype):
+    return _seqmix(x).rms_norm_rows(x, w, eps, out_dtype)
+
+
+def residual_sum_norm(x, ys, scales, gain, eps, out_dtype):
+    return _seqmix(x).residual_sum_norm(x, ys, scales, gain, eps, out_dtype)
+
+
+def row_norm_store(q, k, v, qw, kw, eps, k_cache, v_cache, slot_mapping):
+    return _seqmix(q).row_norm_store(q, k, v, qw, kw, eps, k_cache, v_cache, slot_mapping)
+
+
+def latent_rope_store(q_abs, q, dkv, w, eps, positions, inv_freq, rot_dims, k_cache, v_cache,
+                      slot_mapping):
+    return _seqmix(q).latent_rope_store(q_abs, q, dkv, w, eps, positions, inv_freq, rot_dims,
+                                        k_cache, v_cache, slot_mapping)
+
+
+def xielu(u, ap, aq, out_dtype):
+    return _seqmix(u).xielu(u, ap, aq, out_dtype)
+
+
+def gated_group_norm(o, skip_x, skip_w, z, w, groups, eps, out_dtype):
+    return _seqmix(o).gated_group_norm(o, skip_x, skip_w, z, w, groups, eps, out_dtype)
+
+
+def sigmoid_gate(o, gate, out_dtype):
+    return _seqmix(o).sigmoid_gate(o, gate, out_dtype)

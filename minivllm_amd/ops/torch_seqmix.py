@@ -187,8 +187,12 @@ def unit_norm_store(q, k, eps, k_cache, v_cache, slot_mapping):
 
 
 # ------------------------------------------------------------------ gated delta rule
-def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots):
-    """Short causal convolution + silu on q / k / v (their last taps-1 inputs per sequence live
+def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots,
+                  conv_bias=None, ssd=False):
+    """(``ssd``: the state-space form - the convolution has a bias ``conv_bias`` [C], q and k stay
+    as convolved (no unit vectors, no D^-1/2), beta = softplus(a + dt_bias) is the step size and
+    decay = exp(-exp(A_log) beta); ``b`` is not read.)
+    Short causal convolution + silu on q / k / v (their last taps-1 inputs per sequence live
     in ``conv_state`` [slots, taps-1, Cq+Ck+Cv] fp32 and are replaced by this step's), unit
     vectors for q (times D^-1/2) and k, beta = sigmoid(b), decay = exp(-exp(A_log) softplus(a +
     dt_bias)).  q, k [T,G,D]; v [T,H,E]; b [T,H]; a and dt_bias [T,H] / [H] (a decay per head) or
@@ -213,13 +217,18 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
             full = x[s:e]
         win = full.unfold(0, taps, 1)                                  # [n, C, taps]
         y[s:e] = (win * w[None]).sum(-1)
+    if conv_bias is not None:
+        y = y + conv_bias.float()
     y = F.silu(y)
     cq, ckk = G * D, 2 * G * D
     qn, kn, vv = y[:, :cq].view(T, G, D), y[:, cq:ckk].view(T, G, D), y[:, ckk:].view(T, H, E)
+    sp = F.softplus(a.float() + dt_bias.float())
+    if ssd:
+        decay = torch.exp(-torch.exp(a_log.float()) * sp)
+        return qn.contiguous(), kn.contiguous(), vv.contiguous(), sp, decay
     qn = qn * torch.rsqrt(qn.pow(2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
     kn = kn * torch.rsqrt(kn.pow(2).sum(-1, keepdim=True) + 1e-6)
     beta = torch.sigmoid(b.float())
-    sp = F.softplus(a.float() + dt_bias.float())
     if a.shape[-1] == H:                                                 # one decay per head
         decay = torch.exp(-torch.exp(a_log.float()) * sp)
     else:                                                                # one per head and key channel
@@ -227,9 +236,9 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
     return qn, kn, vv.contiguous(), beta, decay
 
 
-def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
+def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots, correct=True):
     """Per sequence and head, token after token: S <- decay S; u = beta (v - S^T k); S <- S + k
-    u^T; o = S^T q.  ``state`` [slots, H, D, E] fp32 is read (zeros where the sequence starts at
+    u^T; o = S^T q (``correct`` False: u = beta v, the plain gated outer-product update).  ``state`` [slots, H, D, E] fp32 is read (zeros where the sequence starts at
     position 0) and left holding the state after the step.  ``decay`` [T,H] scales a head's whole
     state, [T,H,D] the rows that belong to key channels.  Returns o [T,H,E] fp32."""
     T, G, D = qn.shape
@@ -246,7 +255,7 @@ def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
         S = state[slot].clone() if int(positions[s]) > 0 else torch.zeros(H, D, E)
         for t in range(s, e):
             S = S * (decay[t][:, None, None] if decay.dim() == 2 else decay[t][:, :, None])
-            u = beta[t][:, None] * (vv[t] - torch.einsum("hde,hd->he", S, kh[t]))
+            u = beta[t][:, None] * ((vv[t] - torch.einsum("hde,hd->he", S, kh[t])) if correct else vv[t])
             S = S + kh[t][:, :, None] * u[:, None, :]
             o[t] = torch.einsum("hde,hd->he", S, qh[t])
         state[slot] = S
@@ -407,3 +416,102 @@ def gla_scan(q, k, v, a_raw, a_bias, tau, state, cu_q, positions, slots):
             o[t] = torch.einsum("hde,hd->he", S, qf[t])
         state[slot] = S
     return o
+
+
+# ------------------------------------------------------------------ scaled branches, latent keys
+def rms_norm_rows(x, w, eps, out_dtype):
+    """x [T, n] (rows may be strided, any activation type) / rms * w [n] (fp32 math)."""
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def residual_sum_norm(x, ys, scales, gain, eps, out_dtype):
+    """``x += sum_i scales[i] * ys[i]`` in place on the fp32 stream; with ``gain`` (one number for
+    all coordinates) also returns x / rms(x) * gain, the next layer's input."""
+    for y, s in zip(ys, scales):
+        x.add_(y.float() * float(s))
+    if gain is None:
+        return None
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * float(gain)).to(out_dtype)
+
+
+def _scatter_rows(cache, rows, slot_mapping):
+    bs = cache.shape[1]
+    slots = slot_mapping.long()
+    keep = slots >= 0
+    blk, off = torch.div(slots[keep], bs, rounding_mode="floor"), slots[keep] % bs
+    cache[blk, off] = rows[keep].to(cache.dtype)
+
+
+def row_norm_store(q, k, v, qw, kw, eps, k_cache, v_cache, slot_mapping):
+    """q [T,H,D], k [T,G,D], v [T,G,E] views of a projection output.  With ``qw`` [H*D] / ``kw``
+    [G*D]: the whole q row (all heads at once) is divided by its root mean square and multiplied
+    by qw, in place; the k row likewise with kw on its way into the cache.  Without: k goes in as
+    it is.  v always does.  Rows with slot < 0 store nothing."""
+    T = q.shape[0]
+    kf = k.float()
+    if qw is not None:
+        q.copy_(rms_norm_rows(q.reshape(T, -1), qw, eps, q.dtype).view(q.shape))
+        kf = rms_norm_rows(k.reshape(T, -1), kw, eps, torch.float32).view(k.shape)
+    if k_cache is not None and slot_mapping is not None:
+        _scatter_rows(k_cache, kf, slot_mapping)
+        _scatter_rows(v_cache, v.float(), slot_mapping)
+
+
+def _rotate_half(x, positions, inv_freq, dims):
+    """x [T, ..., n] fp32: entry i < dims/2 is paired with entry i + dims/2 and the pair turned by
+    the fp32 angle position * inv_freq[i]; entries from ``dims`` on pass unchanged."""
+    if dims == 0:
+        return x
+    half = dims // 2
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
+    c, s = torch.cos(ang.double()).float().view(shape), torch.sin(ang.double()).float().view(shape)
+    u, v = x[..., :half], x[..., half:dims]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
+
+
+def latent_rope_store(q_abs, q, dkv, w, eps, positions, inv_freq, rot_dims, k_cache, v_cache,
+                      slot_mapping):
+    """Assembles the queries and cache rows of attention over a shared latent.  ``q_abs`` [H,T,R]:
+    the heads' unrotated query parts carried into the latent's coordinates; ``q`` [T,H,D+P] whose
+    last P entries per head are the part to rotate; ``dkv`` [T,R+P]: the raw latent and one key
+    part shared by all heads.  K cache row = [rmsnorm(latent) * w | rotated key part] (one KV
+    head of R + P), V cache row = the normed latent (R).  Returns the queries [T,H,R+P] =
+    [q_abs | rotated part].  The rotation turns the first ``rot_dims`` of the P entries."""
+    H, T, R = q_abs.shape
+    P = dkv.shape[1] - R
+    D = q.shape[2] - P
+    c = rms_norm_rows(dkv[:, :R], w, eps, torch.float32)
+    kr = _rotate_half(dkv[:, R:].float(), positions, inv_freq, rot_dims)
+    qr = _rotate_half(q[:, :, D:].float(), positions, inv_freq, rot_dims)
+    out = torch.cat([q_abs.transpose(0, 1).float(), qr], -1).to(q.dtype)
+    if k_cache is not None and slot_mapping is not None:
+        _scatter_rows(k_cache, torch.cat([c, kr], -1)[:, None, :], slot_mapping)
+        _scatter_rows(v_cache, c[:, None, :], slot_mapping)
+    return out
+
+
+def xielu(u, ap, aq, out_dtype):
+    """ap z^2 + z/2 for z > 0, aq (e^z - 1 - z) + z/2 otherwise (fp32 math); u may be a strided
+    column block.  Returns a contiguous tensor."""
+    z = u.float()
+    neg = torch.clamp(z, max=0.0)
+    return torch.where(z > 0, ap * z * z + 0.5 * z, aq * (torch.expm1(neg) - neg) + 0.5 * z).to(out_dtype)
+
+
+def gated_group_norm(o, skip_x, skip_w, z, w, groups, eps, out_dtype):
+    """y = (o + skip_w[h] * skip_x) * silu(z) over [T, H*E]; then y is cut into ``groups`` equal
+    consecutive parts, each divided by its own root mean square, times w [H*E].  o, skip_x
+    [T,H,E] fp32; skip_w [H]; z [T, H*E] (strided)."""
+    T, H, E = o.shape
+    y = (o + skip_w.float()[None, :, None] * skip_x).view(T, H * E) * F.silu(z.float())
+    parts = y.view(T, groups, -1)
+    y = (parts * torch.rsqrt(parts.pow(2).mean(-1, keepdim=True) + eps)).view(T, H * E)
+    return (y * w.float()).to(out_dtype)
+
+
+def sigmoid_gate(o, gate, out_dtype):
+    """o [T,H,E] (any strides) * sigmoid(gate [T, H*E]) element by element -> contiguous [T, H*E]."""
+    T = o.shape[0]
+    return (o.float().reshape(T, -1) * torch.sigmoid(gate.float())).to(out_dtype)
