@@ -1,6 +1,9 @@
 // Gated delta rule: preparation of a step's tokens (short causal convolution + silu on q / k / v,
 // unit vectors, beta and decay) and the recurrence itself, for prefill portions and single
 // decode tokens alike.  Everything here is fp32 except the projection outputs it reads.
+// The state-space form (`ssd`: a convolution with bias, q / k as convolved, beta = the step size
+// softplus(a + dt_bias), decay = exp(-exp(A_log) beta)) and the update without the correction
+// term (`DELTA` false: u = beta v) make the same two kernels run a Mamba-2 style mixer.
 //
 // Sequence layout: `cu_q` [B+1] rows of each sequence (null: row b is sequence b), `positions`
 // (a sequence's first row holds the position its portion starts at; 0 = start from zeros),
@@ -22,6 +25,7 @@ template <typename T, int TAPS>
 __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride, int b_off,
                                      const T* __restrict__ a, long a_row, int DC,
                                      const float* __restrict__ conv_w, int taps_rt,
+                                     const float* __restrict__ conv_b, int ssd,
                                      const float* __restrict__ a_log,
                                      const float* __restrict__ dt_bias,
                                      const float* __restrict__ conv_state,
@@ -66,7 +70,7 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride
             float acc[8];
 #pragma unroll
             for (int z = 0; z < 8; ++z) {
-                float a = 0.f;
+                float a = conv_b ? conv_b[c + z] : 0.f;
 #pragma unroll
                 for (int j = 0; j < NT; ++j) a += x[j][z] * w[z][j];
                 acc[z] = siluf_(a);
@@ -77,7 +81,7 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride
         }
     } else
     for (int c = threadIdx.x; c < C; c += blockDim.x) {
-        float acc = 0.f;
+        float acc = conv_b ? conv_b[c] : 0.f;
         for (int j = 0; j < taps; ++j) {             // tap j reads the input `taps-1-j` tokens back
             const int back = taps - 1 - j;
             float x;
@@ -95,17 +99,19 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride
         const float* src = y + hd * D;
         float s = 0.f;
         for (int d = lane; d < D; d += kWave) s += src[d] * src[d];
-        float r = rsqrtf(wave_sum(s) + 1e-6f);
+        float r = ssd ? 1.f : rsqrtf(wave_sum(s) + 1e-6f);
         float* dst;
-        if (hd < G) { r *= rsqrtf((float)D); dst = qn + (t * G + hd) * (long)D; }
+        if (hd < G) { if (!ssd) r *= rsqrtf((float)D); dst = qn + (t * G + hd) * (long)D; }
         else dst = kn + (t * G + hd - G) * (long)D;
         for (int d = lane; d < D; d += kWave) dst[d] = src[d] * r;
     }
-    for (int h = threadIdx.x; h < H; h += blockDim.x)
-        beta[t * H + h] = sigmoidf_(ld(proj + t * row_stride + b_off + h));
+    if (!ssd)
+        for (int h = threadIdx.x; h < H; h += blockDim.x)
+            beta[t * H + h] = sigmoidf_(ld(proj + t * row_stride + b_off + h));
     for (int c = threadIdx.x; c < H * DC; c += blockDim.x) {
-        const float z = ld(a + t * a_row + c) + dt_bias[c];
-        decay[t * (long)(H * DC) + c] = expf(-expf(a_log[c / DC]) * softplusf_(z));
+        const float sp = softplusf_(ld(a + t * a_row + c) + dt_bias[c]);
+        if (ssd) beta[t * H + c] = sp;               // DC == 1: the step size of head c
+        decay[t * (long)(H * DC) + c] = expf(-expf(a_log[c / DC]) * sp);
     }
 }
 
@@ -152,7 +158,7 @@ __global__ void delta_conv_tail_kernel(const T* __restrict__ proj, long row_stri
 // LDS reads (per-lane global loads of these shared vectors were what bound the first version).
 template <int NR> struct ScanChunk { static constexpr int tokens = NR >= 64 ? 8 : 16; };
 
-template <int NR>
+template <int NR, bool DELTA>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                   const float* __restrict__ vv, const float* __restrict__ beta,
@@ -239,16 +245,19 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
             for (int i = 0; i < NR / 4; ++i) { k4[i] = kp[i]; q4[i] = qp[i]; }
             // four partial sums each: a single chain of NR dependent FMAs would be what a step
             // waits for (one wave per SIMD: nobody else fills the gaps)
-            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+            float u = bt * ve;
+            if constexpr (DELTA) {
+                float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
-            for (int i = 0; i < NR / 4; ++i) {
-                d0 += S[4 * i] * k4[i].x; d1 += S[4 * i + 1] * k4[i].y;
-                d2 += S[4 * i + 2] * k4[i].z; d3 += S[4 * i + 3] * k4[i].w;
+                for (int i = 0; i < NR / 4; ++i) {
+                    d0 += S[4 * i] * k4[i].x; d1 += S[4 * i + 1] * k4[i].y;
+                    d2 += S[4 * i + 2] * k4[i].z; d3 += S[4 * i + 3] * k4[i].w;
+                }
+                float dot = (d0 + d1) + (d2 + d3);
+                dot += __shfl_xor(dot, 1, kWave);
+                dot += __shfl_xor(dot, 2, kWave);
+                u = bt * (ve - gd * dot);
             }
-            float dot = (d0 + d1) + (d2 + d3);
-            dot += __shfl_xor(dot, 1, kWave);
-            dot += __shfl_xor(dot, 2, kWave);
-            const float u = bt * (ve - gd * dot);
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int i = 0; i < NR / 4; ++i) {
@@ -272,13 +281,13 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
     }
 }
 
-template <int NR>
+template <int NR, bool DELTA>
 static void launch_scan(dim3 grid, hipStream_t s, const void* qn, const void* kn, const void* vv,
                         const void* beta, const void* decay, void* state, const void* cu_q,
                         const void* positions, const void* slots, void* o, int H, int G, int D, int E) {
     constexpr int CT = ScanChunk<NR>::tokens;
     constexpr int BUF = 2 * CT * 4 * (NR + 4) + CT * 64 + 2 * CT;
-    hipLaunchKernelGGL(delta_scan_kernel<NR>, grid, dim3(256), 2 * BUF * sizeof(float), s,
+    hipLaunchKernelGGL((delta_scan_kernel<NR, DELTA>), grid, dim3(256), 2 * BUF * sizeof(float), s,
                        (const float*)qn, (const float*)kn, (const float*)vv, (const float*)beta,
                        (const float*)decay, (float*)state, (const int*)cu_q, (const int*)positions,
                        (const int*)slots, (float*)o, H, G, D, E);
@@ -287,12 +296,13 @@ static void launch_scan(dim3 grid, hipStream_t s, const void* qn, const void* kn
 extern "C" {
 
 int hyb_delta_prepare(const void* proj, long row_stride, int b_off, const void* a, long a_row,
-                      int DC, const void* conv_w, int taps, const void* a_log, const void* dt_bias, void* conv_state,
+                      int DC, const void* conv_w, int taps, const void* conv_b, int ssd,
+                      const void* a_log, const void* dt_bias, void* conv_state,
                       const void* cu_q, const void* positions, const void* slots,
                       const void* row_seq, void* qn, void* kn, void* vv, void* beta, void* decay,
                       long T_, int B, int H, int G, int D, int E, int dt, hipStream_t s) {
     if (T_ <= 0) return 0;
-    if (taps < 1 || taps > MAX_TAPS || H % G || (DC != 1 && DC != D)) return 1;
+    if (taps < 1 || taps > MAX_TAPS || H % G || (DC != 1 && DC != D) || (ssd && DC != 1)) return 1;
     const int C = 2 * G * D + H * E;
     const size_t lds = 2 * (size_t)G * D * sizeof(float);
     if (lds > 64 * 1024) return 1;
@@ -302,7 +312,8 @@ int hyb_delta_prepare(const void* proj, long row_stride, int b_off, const void* 
     HYB_DISPATCH(dt, hipLaunchKernelGGL((delta_prepare_kernel<T, TAPS>), dim3(T_),                 \
                                         dim3(C >= 2048 && T_ <= 1024 ? 1024 : 256), lds, s,        \
                                         (const T*)proj, row_stride, b_off, (const T*)a, a_row, DC, \
-                                        (const float*)conv_w, taps, (const float*)a_log,           \
+                                        (const float*)conv_w, taps, (const float*)conv_b, ssd,     \
+                                        (const float*)a_log,                                       \
                                         (const float*)dt_bias, (const float*)conv_state,           \
                                         (const int*)cu_q, (const int*)positions, (const int*)slots,\
                                         (const int*)row_seq, (float*)qn, (float*)kn, (float*)vv,   \
@@ -325,11 +336,18 @@ int hyb_delta_prepare(const void* proj, long row_stride, int b_off, const void* 
 
 int hyb_delta_scan(const void* qn, const void* kn, const void* vv, const void* beta,
                    const void* decay, void* state, const void* cu_q, const void* positions,
-                   const void* slots, void* o, int B, int H, int G, int D, int E, hipStream_t s) {
+                   const void* slots, void* o, int B, int H, int G, int D, int E, int correct,
+                   hipStream_t s) {
     if (B <= 0) return 0;
     if (H % G || D > 256) return 1;
     const dim3 grid(B, H, (E + 63) / 64);
-#define SCAN(NR) launch_scan<NR>(grid, s, qn, kn, vv, beta, decay, state, cu_q, positions, slots, o, H, G, D, E)
+#define SCAN(NR)                                                                                       \
+    do {                                                                                               \
+        if (correct) launch_scan<NR, true>(grid, s, qn, kn, vv, beta, decay, state, cu_q, positions,   \
+                                           slots, o, H, G, D, E);                                      \
+        else launch_scan<NR, false>(grid, s, qn, kn, vv, beta, decay, state, cu_q, positions, slots,   \
+                                    o, H, G, D, E);                                                    \
+    } while (0)
     if (D <= 32) SCAN(8);
     else if (D <= 64) SCAN(16);
     else if (D <= 128) SCAN(32);

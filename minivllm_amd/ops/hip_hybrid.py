@@ -50,9 +50,9 @@ _split = _sig("hyb_sink_attention_split", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P
 _split_ok = _lib.hyb_sink_attention_split_ok
 _split_ok.argtypes = [_I, _I]
 _split_ok.restype = _I
-_prep = _sig("hyb_delta_prepare", _P, _L, _I, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P,
-             _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
-_scan = _sig("hyb_delta_scan", _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P)
+_prep = _sig("hyb_delta_prepare", _P, _L, _I, _P, _L, _I, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P,
+             _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
+_scan = _sig("hyb_delta_scan", _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P)
 _cscan = _sig("hyb_channel_delta_scan", _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P)
 _gla = _sig("hyb_gla_scan", _P, _P, _P, _L, _L, _L, _P, _L, _P, _F, _P, _P, _P, _P, _P, _I, _I, _I, _I,
             _I, _P)
@@ -64,6 +64,14 @@ _anm = _sig("hyb_add_normed_mean", _P, _P, _L, _P, _P, _L, _P, _L, _I, _F, _I, _
 _uns = _sig("hyb_unit_norm_store", _P, _P, _L, _F, _P, _P, _P, _L, _I, _I, _I, _I, _P)
 _swi = _sig("hyb_swiglu_route_scale", _P, _L, _P, _P, _L, _I, _I, _I, _I, _P)
 _cap = _sig("hyb_tanh_cap", _P, _L, _F, _I, _P)
+_rsn = _sig("hyb_residual_sum_norm", _P, _P, _P, _P, _I, _F, _P, _L, _I, _F, _I, _P)
+_rnr = _sig("hyb_rms_norm_rows", _P, _L, _P, _P, _L, _I, _F, _I, _P)
+_rns = _sig("hyb_row_norm_store", _P, _P, _P, _L, _P, _P, _F, _P, _P, _P, _L, _I, _I, _I, _I, _P)
+_lrs = _sig("hyb_latent_rope_store", _P, _P, _L, _P, _L, _P, _F, _P, _P, _I, _P, _P, _P, _P, _L, _I,
+            _I, _I, _I, _I, _P)
+_xie = _sig("hyb_xielu", _P, _L, _P, _L, _I, _F, _F, _I, _P)
+_ggn = _sig("hyb_gated_group_norm", _P, _P, _P, _P, _L, _P, _P, _L, _I, _I, _I, _F, _I, _P)
+_sgt = _sig("hyb_sigmoid_gate", _P, _L, _L, _P, _L, _P, _L, _I, _I, _I, _P)
 
 _DT = {torch.bfloat16: 0, torch.float32: 2}
 
@@ -276,7 +284,7 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
 
 # ------------------------------------------------------------------ gated delta rule
 def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots,
-                  row_seq):
+                  row_seq, conv_bias=None, ssd=False):
     T, G, D = q.shape
     H, E = v.shape[1], v.shape[2]
     rs = q.stride(0)
@@ -285,11 +293,13 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
     # q, k, v are the first three column blocks of one projection output, b a view of it; a is a
     # view of it too or a tensor of its own, [T, H] (a decay per head) or [T, H*D] (per key channel)
     assert k.data_ptr() == base + G * D * es and v.data_ptr() == base + 2 * G * D * es
-    assert T == 1 or (k.stride(0) == rs and v.stride(0) == rs and b.stride(0) == rs)
+    assert T == 1 or (k.stride(0) == rs and v.stride(0) == rs and (ssd or b.stride(0) == rs))
     assert a.dtype == q.dtype and a.stride(-1) == 1 and a.shape[-1] in (H, H * D)
     DC = a.shape[-1] // H
-    assert dt_bias.numel() == H * DC
-    b_off = (b.data_ptr() - base) // es
+    assert dt_bias.numel() == H * DC and (not ssd or DC == 1)
+    b_off = 0 if ssd else (b.data_ptr() - base) // es
+    if conv_bias is not None:
+        assert conv_bias.numel() == 2 * G * D + H * E
     dev = q.device
     taps = _f32(conv_w).shape[1]
     assert conv_w.shape[0] == 2 * G * D + H * E
@@ -301,8 +311,8 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
         assert row_seq is not None, "prefill-form steps pass the sequence of each row"
     B = slots.shape[0]
     _check(_prep(base, rs if T > 1 else int(rs or 0), b_off, a.data_ptr(), a.stride(0), DC,
-                 conv_w.data_ptr(), taps, _f32(a_log).data_ptr(),
-                 _f32(dt_bias).data_ptr(), _f32(conv_state).data_ptr(), _ptr(_i32(cu_q)),
+                 conv_w.data_ptr(), taps, _ptr(_f32(conv_bias)) if conv_bias is not None else None,
+                 int(bool(ssd)), _f32(a_log).data_ptr(), _f32(dt_bias).data_ptr(), _f32(conv_state).data_ptr(), _ptr(_i32(cu_q)),
                  _i32(positions).data_ptr(), _i32(slots).data_ptr(),
                  _ptr(_i32(row_seq)) if cu_q is not None else None, qn.data_ptr(), kn.data_ptr(),
                  vv.data_ptr(), beta.data_ptr(), decay.data_ptr(), T, B, H, G, D, E, _dt(q),
@@ -310,13 +320,13 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
     return qn, kn, vv, beta, decay
 
 
-def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
+def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots, correct=True):
     T, G, D = qn.shape
     H, E = vv.shape[1], vv.shape[2]
     assert state.shape[1:] == (H, D, E)
     o = torch.zeros((T, H, E), dtype=torch.float32, device=qn.device)
     if decay.dim() == 3:                 # a decay per head and key channel
-        assert decay.shape == (T, H, D) and decay.is_contiguous()
+        assert decay.shape == (T, H, D) and decay.is_contiguous() and correct
         _check(_cscan(qn.data_ptr(), kn.data_ptr(), vv.data_ptr(), beta.data_ptr(), decay.data_ptr(),
                       _f32(state).data_ptr(), _ptr(_i32(cu_q)), _i32(positions).data_ptr(),
                       _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0], H, G, D, E, _stream()),
@@ -324,8 +334,8 @@ def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
         return o
     _check(_scan(qn.data_ptr(), kn.data_ptr(), vv.data_ptr(), beta.data_ptr(), decay.data_ptr(),
                  _f32(state).data_ptr(), _ptr(_i32(cu_q)), _i32(positions).data_ptr(),
-                 _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0], H, G, D, E, _stream()),
-           "delta_scan")
+                 _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0], H, G, D, E, int(bool(correct)),
+                 _stream()), "delta_scan")
     return o
 
 
@@ -477,3 +487,99 @@ def gla_scan(q, k, v, a_raw, a_bias, tau, state, cu_q, positions, slots):
                 _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0], H, D, E, _dt(q), _stream()),
            "gla_scan")
     return o
+
+
+# ------------------------------------------------------------------ scaled branches, latent keys
+def rms_norm_rows(x, w, eps, out_dtype):
+    T, n = x.shape
+    assert x.stride(1) == 1 and x.dtype == out_dtype and w.numel() == n
+    out = torch.empty((T, n), dtype=out_dtype, device=x.device)
+    _check(_rnr(x.data_ptr(), _rows(x), _f32(w).data_ptr(), out.data_ptr(), T, n, eps, _dt(x),
+                _stream()), "rms_norm_rows")
+    return out
+
+
+def residual_sum_norm(x, ys, scales, gain, eps, out_dtype):
+    x = _f32(x)
+    T, W = x.shape
+    ys = list(ys)
+    assert len(ys) <= 4 and len(ys) == len(scales), "at most four branches are added per call"
+    for y in ys:
+        assert y.shape == x.shape and y.stride(1) == 1 and y.dtype == out_dtype
+    h = torch.empty((T, W), dtype=out_dtype, device=x.device) if gain is not None else None
+    if h is None and not ys:
+        return None
+    n = len(ys)
+    ptrs = (ctypes.c_void_p * 4)(*[y.data_ptr() for y in ys], *([None] * (4 - n)))
+    strides = (ctypes.c_long * 4)(*[_rows(y) for y in ys], *([0] * (4 - n)))
+    sc = (ctypes.c_float * 4)(*[float(v) for v in scales], *([0.0] * (4 - n)))
+    _check(_rsn(x.data_ptr(), ptrs, strides, sc, n, float(gain) if gain is not None else 0.0,
+                _ptr(h), T, W, eps, _DT[out_dtype], _stream()), "residual_sum_norm")
+    return h
+
+
+def row_norm_store(q, k, v, qw, kw, eps, k_cache, v_cache, slot_mapping):
+    T, H, D = q.shape
+    G, E = v.shape[1], v.shape[2]
+    rs = q.stride(0)
+    assert (T == 1 or (k.stride(0) == rs and v.stride(0) == rs)) and q.stride(1) == D \
+        and k.stride(1) == D and v.stride(1) == E and q.stride(2) == 1 and k.stride(2) == 1 \
+        and v.stride(2) == 1, "q / k / v must be views of one projection output"
+    assert (qw is None) == (kw is None)
+    if qw is not None:
+        assert qw.numel() == H * D and kw.numel() == G * D
+    if k_cache is not None:
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype \
+            and k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, E)
+    _check(_rns(q.data_ptr(), k.data_ptr(), v.data_ptr(), rs, _ptr(_f32(qw)) if qw is not None else None,
+                _ptr(_f32(kw)) if kw is not None else None, eps, _ptr(k_cache), _ptr(v_cache),
+                _ptr(_i32(slot_mapping)), T, H * D, G * D, G * E, _dt(q), _stream()), "row_norm_store")
+
+
+def latent_rope_store(q_abs, q, dkv, w, eps, positions, inv_freq, rot_dims, k_cache, v_cache,
+                      slot_mapping):
+    H, T, R = q_abs.shape
+    P = dkv.shape[1] - R
+    D = q.shape[2] - P
+    assert q_abs.is_contiguous() and q_abs.dtype == q.dtype and dkv.dtype == q.dtype
+    assert q.shape[:2] == (T, H) and q.stride(2) == 1 and q.stride(1) == D + P and dkv.stride(1) == 1
+    assert w.numel() == R and inv_freq.numel() * 2 == rot_dims
+    if k_cache is not None:
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype \
+            and k_cache.shape[2:] == (1, R + P) and v_cache.shape[2:] == (1, R)
+    out = torch.empty((T, H, R + P), dtype=q.dtype, device=q.device)
+    _check(_lrs(q_abs.data_ptr(), q.data_ptr(), _rows(q), dkv.data_ptr(), _rows(dkv),
+                _f32(w).data_ptr(), eps, _i32(positions).data_ptr(), _f32(inv_freq).data_ptr(),
+                int(rot_dims), _ptr(k_cache), _ptr(v_cache), _ptr(_i32(slot_mapping)), out.data_ptr(),
+                T, H, D, P, R, _dt(q), _stream()), "latent_rope_store")
+    return out
+
+
+def xielu(u, ap, aq, out_dtype):
+    T, n = u.shape
+    assert u.stride(1) == 1 and u.dtype == out_dtype
+    act = torch.empty((T, n), dtype=out_dtype, device=u.device)
+    _check(_xie(u.data_ptr(), _rows(u), act.data_ptr(), T, n, float(ap), float(aq), _dt(u),
+                _stream()), "xielu")
+    return act
+
+
+def gated_group_norm(o, skip_x, skip_w, z, w, groups, eps, out_dtype):
+    T, H, E = o.shape
+    assert skip_x.shape == o.shape and z.shape == (T, H * E) and z.stride(1) == 1 \
+        and z.dtype == out_dtype and w.numel() == H * E and skip_w.numel() == H
+    out = torch.empty((T, H * E), dtype=out_dtype, device=o.device)
+    _check(_ggn(_f32(o).data_ptr(), _f32(skip_x).data_ptr(), _f32(skip_w).data_ptr(), z.data_ptr(),
+                _rows(z), _f32(w).data_ptr(), out.data_ptr(), T, H, E, int(groups), eps,
+                _DT[out_dtype], _stream()), "gated_group_norm")
+    return out
+
+
+def sigmoid_gate(o, gate, out_dtype):
+    T, H, E = o.shape
+    assert o.stride(2) == 1 and gate.shape == (T, H * E) and gate.stride(1) == 1 \
+        and o.dtype == out_dtype and gate.dtype == out_dtype
+    out = torch.empty((T, H * E), dtype=out_dtype, device=o.device)
+    _check(_sgt(o.data_ptr(), o.stride(0), o.stride(1), gate.data_ptr(), _rows(gate), out.data_ptr(),
+                T, H, E, _dt(o), _stream()), "sigmoid_gate")
+    return out
