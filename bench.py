@@ -333,6 +333,32 @@ def pelenex_model(size: str, vocab: int = 32768, experts: int = 4, top: int = 2,
                                     "layers": layers, "max_position": 8192}, name=f"pelenex-{size}")
 
 
+def kidupel_model(size: str, vocab: int = 32768, window: int = 512):
+    """Kidupel configuration of the same width, number of layer runs, head geometry and
+    feed-forward parameters per token as ``hybrid_models(size)``: six layers (parallel mixer =
+    windowed gated attention + state-space duality, latent attention, whole-projection-normed
+    attention, twice) of which the second and third run twice, i.e. eight layer runs; dense
+    xIELU feed-forward with 2 * ff = 3 * intermediate; state-space mixer with inner size 2 W in
+    heads of 64, state 128 (the usual Mamba-2 proportions); latent of 128 + a rotated part of 128."""
+    from minivllm_amd.models.kidupel import KidupelConfig
+    W, L, H, G, D, inter = HYBRID_SIZES[size]
+    mlp = {"kind": "dense", "ff": 3 * inter // 2 // 64 * 64}
+    mask = {"size": window}
+    kinds = [("parallel", {"left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+                                    "mask": mask},
+                           "left_scale": 1.0, "right_scale": 1.0,
+                           "right": {"heads": 2 * W // 64, "groups": 8, "state": 128, "vdim": 64,
+                                     "conv": 4, "norm_groups": 8}}),
+             ("latent_attention", {"heads": H, "dim": D, "rot_dim": 128, "vdim": D, "kv_rank": 128,
+                                   "q_rank": 3 * W // 8, "scale": (D + 128) ** -0.5, "mask": mask,
+                                   "rot": {"base": 10000.0, "dims": 128}}),
+             ("attention", {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": 1.0, "mask": mask})]
+    layers = [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": mlp} for i in range(L - 2)]
+    return KidupelConfig.from_dict({"architecture": "Kidupel", "vocab": vocab, "width": W,
+                                    "norm": {"eps": 1e-6}, "layers": layers,
+                                    "loop": {"start": 1, "stop": 3, "times": 2}}, name=f"kidupel-{size}")
+
+
 def hybrid_comparison(args) -> dict:
     """Prefill and decode throughput of the hybrid families next to the dense decoder of the same
     size, one GPU, same engine path as the headline measurement (``bench_model``).
@@ -340,6 +366,8 @@ def hybrid_comparison(args) -> dict:
     closest relative: attention + delta rule + routed experts around a fp32 stream) and dense."""
     if args.family == "pelenex":
         return pelenex_comparison(args)
+    if args.family == "kidupel":
+        return kidupel_comparison(args)
     out = {"metric": "prefill / decode tok/s, hybrid (attention + delta rule + routed experts) "
                      "next to the dense decoder of equal size",
            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -385,6 +413,34 @@ def pelenex_comparison(args) -> dict:
             if all(n in row and k in row[n] for n in ("pelenex", "natilix", "dense")):
                 row[f"pelenex_over_natilix_{k}"] = round(row["pelenex"][k] / row["natilix"][k], 3)
                 row[f"pelenex_over_dense_{k}"] = round(row["pelenex"][k] / row["dense"][k], 3)
+        out["sizes"][size] = row
+    return out
+
+
+def kidupel_comparison(args) -> dict:
+    out = {"metric": "prefill / decode tok/s, Kidupel (windowed gated attention + state-space "
+                     "duality, latent attention, whole-projection-normed attention, looped layers, "
+                     "xIELU feed-forward) next to Pelenex and the dense decoder of equal size",
+           "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "dtype": "bf16", "data": "synthetic random token prompts, random-init weights",
+           "config": {"seq_len": args.seq_len, "decode_batch": args.batch,
+                      "prefill_tokens_per_step": args.prefill_tokens, "kv_block_size": args.block_size},
+           "sizes": {}}
+    keep = ("prefill_tok_s", "prefill_ms_per_step", "decode_tok_s", "decode_ms_per_step",
+            "hipgraph_captured", "init_s")
+    for size in args.hybrid.split(","):
+        _, dense = hybrid_models(size)
+        row = {}
+        for name, make in (("kidupel", lambda: kidupel_model(size)), ("pelenex", lambda: pelenex_model(size)),
+                           ("dense", lambda: dense)):
+            if args.only and name != args.only:
+                continue                         # (a kernel trace of one model)
+            r = bench_model(args, make(), 0, 1)
+            row[name] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items() if k in keep}
+        for k in ("prefill_tok_s", "decode_tok_s"):
+            if all(n in row and k in row[n] for n in ("kidupel", "pelenex", "dense")):
+                row[f"kidupel_over_pelenex_{k}"] = round(row["kidupel"][k] / row["pelenex"][k], 3)
+                row[f"kidupel_over_dense_{k}"] = round(row["kidupel"][k] / row["dense"][k], 3)
         out["sizes"][size] = row
     return out
 
@@ -688,11 +744,11 @@ def main():
                          "launch floor of a real N-GPU run; NOT a scaling number)")
     ap.add_argument("--p2p", action="store_true",
                     help="with --tp-shard: all-reduces by the peer-to-peer kernels in loop-back form")
-    ap.add_argument("--family", default="natilix", choices=["natilix", "pelenex"],
+    ap.add_argument("--family", default="natilix", choices=["natilix", "pelenex", "kidupel"],
                     help="with --hybrid: which hybrid family is measured (pelenex: next to natilix "
-                         "and dense)")
-    ap.add_argument("--only", default="", choices=["", "pelenex", "natilix", "dense"],
-                    help="with --hybrid --family pelenex: measure this one model only")
+                         "and dense; kidupel: next to pelenex and dense)")
+    ap.add_argument("--only", default="", choices=["", "kidupel", "pelenex", "natilix", "dense"],
+                    help="with --hybrid --family pelenex / kidupel: measure this one model only")
     ap.add_argument("--hybrid", default="",
                     help="instead of the headline workload: the hybrid family (Natilix) next to "
                          "the dense decoder of equal size; comma-separated sizes of "

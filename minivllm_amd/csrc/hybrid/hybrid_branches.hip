@@ -150,15 +150,43 @@ __global__ void latent_rope_store_kernel(const T* __restrict__ q_abs, const T* _
     }
 }
 
+// eight consecutive elements narrowed from fp32 and stored as one run (16 bytes of bfloat16, two
+// 16-byte stores of float); the address must be aligned to the run
+template <typename T> __device__ __forceinline__ void store_run8(T* p, const float* v);
+template <> __device__ __forceinline__ void store_run8<float>(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+template <> __device__ __forceinline__ void store_run8<bf16_t>(bf16_t* p, const float* v) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const __bf16 lo = (__bf16)v[2 * i], hi = (__bf16)v[2 * i + 1];
+        w[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+    }
+    *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__device__ __forceinline__ float xielu_(float z, float above, float below) {
+    return z > 0.f ? above * z * z + 0.5f * z : below * (expm1f(z) - z) + 0.5f * z;
+}
+
 // act = above z^2 + z/2 (z > 0);  below (e^z - 1 - z) + z/2 (z <= 0).  u rows strided, act dense.
-template <typename T>
+// VEC consecutive columns per thread (VEC = 8: rows and row starts are whole 16-byte runs).
+template <typename T, int VEC>
 __global__ void xielu_kernel(const T* __restrict__ u, long u_stride, T* __restrict__ act, int n,
                              float above, float below) {
     const long t = blockIdx.y;
-    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < n; c += gridDim.x * blockDim.x) {
-        const float z = ld(u + t * u_stride + c);
-        const float y = z > 0.f ? above * z * z + 0.5f * z : below * (expm1f(z) - z) + 0.5f * z;
-        st(act + t * (long)n + c, y);
+    for (int c = (blockIdx.x * blockDim.x + threadIdx.x) * VEC; c < n; c += gridDim.x * blockDim.x * VEC) {
+        if constexpr (VEC == 8) {
+            float z[8];
+            load_run<T, 8>(u + t * u_stride + c, z);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) z[j] = xielu_(z[j], above, below);
+            store_run8<T>(act + t * (long)n + c, z);
+        } else {
+            st(act + t * (long)n + c, xielu_(ld(u + t * u_stride + c), above, below));
+        }
     }
 }
 
@@ -190,15 +218,24 @@ __global__ void gated_group_norm_kernel(const float* __restrict__ o, const float
 }
 
 // out[t, h*E + e] = o[t, h, e] * sigmoid(gate[t, h*E + e]); o with strides (o_t, o_h, 1).
-template <typename T>
+template <typename T, int VEC>
 __global__ void sigmoid_gate_kernel(const T* __restrict__ o, long o_t, long o_h,
                                     const T* __restrict__ gate, long gate_stride,
                                     T* __restrict__ out, int H, int E) {
     const long t = blockIdx.y;
     const int n = H * E;
-    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < n; c += gridDim.x * blockDim.x) {
+    for (int c = (blockIdx.x * blockDim.x + threadIdx.x) * VEC; c < n; c += gridDim.x * blockDim.x * VEC) {
         const int hh = c / E, e = c - hh * E;
-        st(out + t * (long)n + c, ld(o + t * o_t + hh * o_h + e) * sigmoidf_(ld(gate + t * gate_stride + c)));
+        if constexpr (VEC == 8) {                       // E % 8 == 0: a run stays inside one head
+            float a[8], g[8];
+            load_run<T, 8>(o + t * o_t + hh * o_h + e, a);
+            load_run<T, 8>(gate + t * gate_stride + c, g);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) a[j] *= sigmoidf_(g[j]);
+            store_run8<T>(out + t * (long)n + c, a);
+        } else {
+            st(out + t * (long)n + c, ld(o + t * o_t + hh * o_h + e) * sigmoidf_(ld(gate + t * gate_stride + c)));
+        }
     }
 }
 
@@ -265,16 +302,25 @@ int hyb_latent_rope_store(const void* q_abs, const void* q, long q_row, const vo
     return HYB_LAUNCH_OK();
 }
 
+// rows of n elements, `stride` apart, can be walked in aligned runs of eight
+static inline bool runs_of_8(const void* p, long stride, int n, int dt) {
+    return n % 8 == 0 && stride % 8 == 0 && (size_t)p % 16 == 0;
+}
+
 int hyb_xielu(const void* u, long u_stride, void* act, long T_, int n, float above, float below,
               int dt, hipStream_t s) {
     if (T_ <= 0 || n <= 0) return 0;
-    const int need = (n + 255) / 256;
+    const bool vec = runs_of_8(u, u_stride, n, dt) && runs_of_8(act, n, n, dt);
+    const int need = (n / (vec ? 8 : 1) + 255) / 256;
     const int bx = need > 64 ? 64 : need;
     for (long t0 = 0; t0 < T_; t0 += 65535) {          // blockIdx.y holds at most 65535 rows
         const long nrow = T_ - t0 < 65535 ? T_ - t0 : 65535;
-        HYB_DISPATCH(dt, hipLaunchKernelGGL(xielu_kernel<T>, dim3(bx, nrow), dim3(256), 0, s,
-                                            (const T*)u + t0 * u_stride, u_stride,
-                                            (T*)act + t0 * (long)n, n, above, below));
+#define XIE(VEC)                                                                                   \
+        HYB_DISPATCH(dt, hipLaunchKernelGGL((xielu_kernel<T, VEC>), dim3(bx, nrow), dim3(256), 0, s, \
+                                            (const T*)u + t0 * u_stride, u_stride,                 \
+                                            (T*)act + t0 * (long)n, n, above, below))
+        if (vec) XIE(8); else XIE(1);
+#undef XIE
     }
     return HYB_LAUNCH_OK();
 }
@@ -297,14 +343,19 @@ int hyb_gated_group_norm(const void* o, const void* x, const void* skip, const v
 int hyb_sigmoid_gate(const void* o, long o_t, long o_h, const void* gate, long gate_stride,
                      void* out, long T_, int H, int E, int dt, hipStream_t s) {
     if (T_ <= 0 || H * E <= 0) return 0;
-    const int need = (H * E + 255) / 256;
+    const bool vec = E % 8 == 0 && o_h % 8 == 0 && runs_of_8(o, o_t, E, dt) &&
+                     runs_of_8(gate, gate_stride, H * E, dt) && runs_of_8(out, H * E, H * E, dt);
+    const int need = (H * E / (vec ? 8 : 1) + 255) / 256;
     const int bx = need > 64 ? 64 : need;
     for (long t0 = 0; t0 < T_; t0 += 65535) {
         const long nrow = T_ - t0 < 65535 ? T_ - t0 : 65535;
-        HYB_DISPATCH(dt, hipLaunchKernelGGL(sigmoid_gate_kernel<T>, dim3(bx, nrow), dim3(256), 0, s,
-                                            (const T*)o + t0 * o_t, o_t, o_h,
-                                            (const T*)gate + t0 * gate_stride, gate_stride,
-                                            (T*)out + t0 * (long)(H * E), H, E));
+#define SGT(VEC)                                                                                   \
+        HYB_DISPATCH(dt, hipLaunchKernelGGL((sigmoid_gate_kernel<T, VEC>), dim3(bx, nrow), dim3(256), \
+                                            0, s, (const T*)o + t0 * o_t, o_t, o_h,                \
+                                            (const T*)gate + t0 * gate_stride, gate_stride,        \
+                                            (T*)out + t0 * (long)(H * E), H, E))
+        if (vec) SGT(8); else SGT(1);
+#undef SGT
     }
     return HYB_LAUNCH_OK();
 }

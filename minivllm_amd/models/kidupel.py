@@ -140,6 +140,19 @@ def _take(w: dict, key: str, shape, where: str) -> torch.Tensor:
     return t
 
 
+def _pad8(rows: List[torch.Tensor], bias: Optional[List[torch.Tensor]] = None) -> int:
+    """Appends zero rows so that the next block of the fused projection starts at a column that is
+    a multiple of eight (kernels read blocks in aligned 16-byte runs when they can).  Returns the
+    number of rows now in ``rows``."""
+    n = sum(r.shape[0] for r in rows)
+    pad = -n % 8
+    if pad:
+        rows.append(torch.zeros(pad, rows[0].shape[1], dtype=rows[0].dtype))
+        if bias is not None:
+            bias.append(torch.zeros(pad, dtype=bias[0].dtype))
+    return n + pad
+
+
 def _window(m: dict) -> int:
     return int((m.get("mask") or {}).get("size", 0))
 
@@ -177,6 +190,7 @@ class KidupelParallelMixer(nn.Module):
         H, G, D, E = a.num_heads, a.num_kv_heads, a.head_dim, a.v_head_dim
         nl = sum(self.left_sizes)
         q, k, v, g = proj[:, :nl].split(self.left_sizes, dim=-1)
+        nl += -nl % 8                                   # the state-space block starts on a run of 8
         q = q.view(T, H, D)
         ops.row_norm_store(q, k.view(T, G, D), v.view(T, G, E), None, None, 0.0, a.k_cache,
                            a.v_cache, get_context().slot_mapping)
@@ -190,6 +204,7 @@ class KidupelParallelMixer(nn.Module):
         rows = [_take(w, "left." + k, (n, W), where) for k, n in
                 (("q", H * D), ("k", G * D), ("v", G * E), ("g", H))]
         self.left_o = _param(_take(w, "left.o", (W, H * E), where), like)
+        _pad8(rows)
         Hs, Gs, N, Es = s.num_heads, s.groups, s.state_size, s.v_head_dim
         inner, gn = Hs * Es, Gs * N
         # checkpoint order of the input projection: z, x, B, C, dt; of the convolution: x, B, C.
@@ -348,7 +363,7 @@ class KidupelLayer(nn.Module):
         proj = F.linear(h, self.in_proj, self.in_bias)
         ys = self.mix(proj[:, :self.mix_rows], h, out_dtype, which)
         if self.ff:
-            ys.append((F.linear(self.act(proj[:, self.mix_rows:], out_dtype), self.down), 1.0))
+            ys.append((F.linear(self.act(proj[:, self.mix_rows:self.mix_rows + self.ff], out_dtype), self.down), 1.0))
         return ys
 
     def load(self, w: dict, where: str, like) -> None:
@@ -358,7 +373,7 @@ class KidupelLayer(nn.Module):
         rows, bias = self.mix.load(mw, where + "mix.", like)
         if mw:
             raise KeyError(f"checkpoint tensor {where}mix.{next(iter(mw))} has no parameter")
-        self.mix_rows = sum(r.shape[0] for r in rows)
+        self.mix_rows = _pad8(rows, bias) if self.ff else sum(r.shape[0] for r in rows)
         if self.ff:
             rows.append(_take(w, "mlp.up", (self.ff, W), where))
             self.down = _param(_take(w, "mlp.down", (W, self.ff), where), like)
@@ -367,6 +382,7 @@ class KidupelLayer(nn.Module):
                 bias.append(torch.zeros(self.ff, dtype=bias[0].dtype))
         if w:
             raise KeyError(f"checkpoint tensor {where}{next(iter(w))} has no parameter")
+        _pad8(rows, bias)                               # row stride of the output: whole runs of 8
         self.in_proj = _param(torch.cat(rows, 0), like)
         self.in_bias = _param(torch.cat(bias, 0), like) if bias is not None else None
 
