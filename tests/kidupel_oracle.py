@@ -38,7 +38,7 @@ def gelu_tanh(z):
 
 
 def scalar_norm(x, g, eps):
-    """RMS norm whose gain is one number for all coordinates."""
+    """RMS norm with a single scalar gain."""
     return rms(x, eps) * float(g)
 
 
