@@ -29,6 +29,9 @@ struct KeyRule {
     int window;             // 0: every earlier key is visible
     int keep_first;
     const float* slopes;    // [H] or null
+    int v_stride;           // elements from one (slot, KV head) value row to the next: E for a dense
+                            // V cache, more when the value rows are the leading part of wider rows
+                            // (values stored inside the key rows: v_cache then points into k_cache)
 };
 
 // The visible keys of a query that sees `ctx` keys without a window (its position is ctx - 1), as
@@ -171,8 +174,8 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
                 const int r = c / E, e = c - r * E;
                 float o = acc[a] * stat[r];
                 const float* pr = ps + r * TILE;
-                const T* vb = v_cache + (long)g * E + e;
-                for (int jj = 0; jj < n; ++jj) o += pr[jj] * ld(vb + rowbase[jj] * (long)(G * E));
+                const T* vb = v_cache + (long)g * rule.v_stride + e;
+                for (int jj = 0; jj < n; ++jj) o += pr[jj] * ld(vb + rowbase[jj] * (long)(G * rule.v_stride));
                 acc[a] = o;
             }
         }
@@ -323,7 +326,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                 float v4[4] = {0.f, 0.f, 0.f, 0.f};
                 if (j < wg_ctx) {
                     const long slot = (long)table[j / block_size] * block_size + j % block_size;
-                    Vec4<T>::load(v_cache + (slot * G + g) * (long)E + c, v4);
+                    Vec4<T>::load(v_cache + (slot * G + g) * (long)rule.v_stride + c, v4);
                 }
                 float* dst = Vs + key * EP + c;
                 dst[0] = v4[0]; dst[1] = v4[1]; dst[2] = v4[2]; dst[3] = v4[3];
@@ -334,7 +337,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                 float v = 0.f;
                 if (j < wg_ctx) {
                     const long slot = (long)table[j / block_size] * block_size + j % block_size;
-                    v = ld(v_cache + (slot * G + g) * (long)E + c);
+                    v = ld(v_cache + (slot * G + g) * (long)rule.v_stride + c);
                 }
                 Vs[key * EP + c] = v;
             }
@@ -417,7 +420,7 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
                         int seq0, int max_q, int H, int G, int D, int E, int esize,
                         KeyRule rule, hipStream_t s) {
     const int vec_k = (D % 4 == 0) && ((size_t)k_cache % 16 == 0);
-    const int vec_v = (E % 4 == 0) && ((size_t)v_cache % 16 == 0);
+    const int vec_v = (E % 4 == 0) && (rule.v_stride % 4 == 0) && ((size_t)v_cache % 16 == 0);
     const dim3 grid(nseq, (max_q + 127) / 128, H);
 #define TILES_LAUNCH(QK16, lds)                                                                   \
     hipLaunchKernelGGL((sink_attention_tiles_kernel<T, DP, EP, QK16>), grid, dim3(256), lds, s,   \
@@ -496,8 +499,8 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
         float kf[2][EPL], vf[2][VPL];
         load_run<T, EPL>(k_cache + (slot * G + g) * (long)D + lane16 * EPL, kf[0]);
         load_run<T, EPL>(k_cache + (slot2 * G + g) * (long)D + lane16 * EPL, kf[1]);
-        load_run<T, VPL>(v_cache + (slot * G + g) * (long)E + lane16 * VPL, vf[0]);
-        load_run<T, VPL>(v_cache + (slot2 * G + g) * (long)E + lane16 * VPL, vf[1]);
+        load_run<T, VPL>(v_cache + (slot * G + g) * (long)rule.v_stride + lane16 * VPL, vf[0]);
+        load_run<T, VPL>(v_cache + (slot2 * G + g) * (long)rule.v_stride + lane16 * VPL, vf[1]);
 #pragma unroll
         for (int x = 0; x < 2; ++x) {
             if (x == 1 && !two) break;
@@ -610,10 +613,11 @@ int hyb_sink_attention_split(const void* q, long q_row, long q_head, const void*
                              int block_size, const void* context_lens, const void* sink,
                              const void* gate, long gate_row, void* out, void* ws, float scale,
                              int B, int H, int G, int D, int E, int splits, int window,
-                             int keep_first, const void* slopes, int dt, hipStream_t s) {
-    const KeyRule rule{window, keep_first, (const float*)slopes};
+                             int keep_first, const void* slopes, int v_stride, int dt, hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E};
     if (B <= 0) return 0;
     if (G <= 0 || H % G || splits < 1 || !hyb_sink_attention_split_ok(D, E)) return 1;
+    if (rule.v_stride < E || rule.v_stride % 8) return 1;      // 16-byte runs of a value row
     if (((size_t)k_cache | (size_t)v_cache | (size_t)q) % 16 || (q_row * (dt == 0 ? 2 : 4)) % 16) return 1;
 #define SPLIT_ARGS q, q_row, q_head, k_cache, v_cache, block_tables, max_blocks, block_size, \
                    context_lens, sink, gate, gate_row, out, ws, scale, B, H, G, splits, rule, s
@@ -643,10 +647,11 @@ int hyb_sink_attention_tiles(const void* q, long q_row, long q_head, const void*
                              int block_size, const void* cu_q, const void* positions,
                              const void* sink, const void* gate, long gate_row, void* out,
                              float scale, int nseq, int seq0, int max_q, int H, int G, int D,
-                             int E, int window, int keep_first, const void* slopes, int dt,
-                             hipStream_t s) {
-    const KeyRule rule{window, keep_first, (const float*)slopes};
+                             int E, int window, int keep_first, const void* slopes, int v_stride,
+                             int dt, hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E};
     if (nseq <= 0 || max_q <= 0) return 0;
+    if (rule.v_stride < E) return 1;
     if (G <= 0 || H % G || !hyb_sink_attention_tiles_ok(D, E)) return 1;
 #define TILES_ARGS q, q_row, q_head, k_cache, v_cache, block_tables, max_blocks, block_size, cu_q, \
                    positions, sink, gate, gate_row, out, scale, nseq, seq0, max_q, H, G, D, E
@@ -675,9 +680,11 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
                             int block_size, const void* row_seq, const void* lens, int len_add,
                             const void* sink, const void* gate, long gate_row, void* out,
                             float scale, long rows, int H, int G, int D, int E, int seq_base,
-                            int window, int keep_first, const void* slopes, int dt, hipStream_t s) {
-    const KeyRule rule{window, keep_first, (const float*)slopes};
+                            int window, int keep_first, const void* slopes, int v_stride, int dt,
+                            hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E};
     if (rows <= 0) return 0;
+    if (rule.v_stride < E) return 1;
     if (G <= 0 || H % G || RC * E > NACC * TILE || D > 1024) return 1;
     const int R = H / G, chunks = (R + RC - 1) / RC;
     const size_t lds = (RC * D + RC * TILE + 4 * RC + 3 * RC + 2) * sizeof(float) + TILE * sizeof(long);

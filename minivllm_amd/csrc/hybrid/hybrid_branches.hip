@@ -90,7 +90,8 @@ __global__ void row_norm_store_kernel(T* __restrict__ q, const T* __restrict__ k
     for (int c = threadIdx.x; c < nv; c += blockDim.x) st(v_cache + slot * nv + c, ld(vr + c));
 }
 
-// Per token: c = rmsnorm(dkv[0:R]) * w;  K cache row = [c | rot(dkv[R:R+P])], V cache row = c;
+// Per token: c = rmsnorm(dkv[0:R]) * w;  K cache row = [c | rot(dkv[R:R+P])], V cache row = c
+// (when a separate V cache is given);
 // out[t, h] = [q_abs[h, t, 0:R] | rot(q[t, h, D:D+P])].  rot: entry i < dims/2 pairs with entry
 // i + dims/2, angle = position * inv_freq[i] (fp32 product), entries from dims on unchanged.
 template <typename T>
@@ -125,7 +126,7 @@ __global__ void latent_rope_store_kernel(const T* __restrict__ q_abs, const T* _
         for (int c = threadIdx.x; c < R; c += blockDim.x) {
             const float a = ld(lr + c) * r * w[c];
             st(k_cache + slot * DK + c, a);
-            st(v_cache + slot * R + c, a);
+            if (v_cache) st(v_cache + slot * R + c, a);   // null: values are read from the key rows
         }
         for (int i = threadIdx.x; i < P; i += blockDim.x) {
             float a;

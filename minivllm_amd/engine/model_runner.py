@@ -601,7 +601,8 @@ class ModelRunner:
         m = self.cfg.model
         itemsize = torch.empty((), dtype=self.kv_dtype).element_size()
         if self.hybrid:
-            return max(1, sum(self.block_size * a.num_kv_heads * (a.head_dim + a.v_head_dim) * itemsize
+            return max(1, sum(self.block_size * a.num_kv_heads * itemsize
+                              * (a.head_dim + (0 if getattr(a, "value_in_key", False) else a.v_head_dim))
                               for a in self.model.attention_layers()))
         return (2 * m.num_layers * self.block_size * (m.num_kv_heads // self.tp)
                 * m.head_dim * itemsize)
@@ -661,14 +662,18 @@ class ModelRunner:
 
     def _allocate_hybrid_caches(self) -> None:
         """One K and one V allocation per attention layer (their head sizes may differ from
-        layer to layer and between K and V), logical [block, token, kv head, d]; per recurrent
+        layer to layer and between K and V; a layer whose values are part of its key rows gets a
+        view instead of a V allocation), logical [block, token, kv head, d]; per recurrent
         layer one fp32 row per state slot of whatever the layer's ``state_spec`` lists (matrix
         state, normaliser, running maximum, convolution tail, ...)."""
         n, bs = self.num_kv_blocks, self.block_size
         self.kv_cache = []
         for a in self.model.attention_layers():
             a.k_cache = torch.zeros(n, bs, a.num_kv_heads, a.head_dim, dtype=self.kv_dtype, device=self.device)
-            a.v_cache = torch.zeros(n, bs, a.num_kv_heads, a.v_head_dim, dtype=self.kv_dtype, device=self.device)
+            if getattr(a, "value_in_key", False):      # values = leading entries of the key rows
+                a.v_cache = a.k_cache[..., :a.v_head_dim]
+            else:
+                a.v_cache = torch.zeros(n, bs, a.num_kv_heads, a.v_head_dim, dtype=self.kv_dtype, device=self.device)
             self.kv_cache.append((a.k_cache, a.v_cache))
         for d in self.model.state_layers():
             for attr, shape in d.state_spec():

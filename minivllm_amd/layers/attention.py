@@ -170,12 +170,17 @@ class SinkAttention(nn.Module):
     Options, each a constructor argument: ``sink=False`` - an ordinary softmax (no extra term);
     ``window`` > 0 - a query at position i sees key j <= i only when i - j < window or
     j < keep_first (the first tokens stay visible at their true positions); ``distance_slopes``
-    [H] - slope_h * (i - j) is taken off the score of key j."""
+    [H] - slope_h * (i - j) is taken off the score of key j; ``value_in_key`` - a token's value is
+    the leading ``v_head_dim`` entries of its key row, so the engine allocates no V cache and
+    ``v_cache`` is a view into ``k_cache``."""
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
                  scale: float, sink: bool = True, window: int = 0, keep_first: int = 0,
-                 distance_slopes: Optional[torch.Tensor] = None):
+                 distance_slopes: Optional[torch.Tensor] = None, value_in_key: bool = False):
         super().__init__()
+        if value_in_key and v_head_dim > head_dim:
+            raise ValueError("values inside the key rows cannot be longer than the keys")
+        self.value_in_key = bool(value_in_key)
         self.num_heads, self.num_kv_heads = num_heads, num_kv_heads
         self.head_dim, self.v_head_dim, self.scale = head_dim, v_head_dim, scale
         self.window, self.keep_first = int(window), int(keep_first)
@@ -227,7 +232,8 @@ class LatentAttention(nn.Module):
     this is attention with ONE key/value head whose key row is [c | r] (R + P) and whose value row
     is c (R), run by ``SinkAttention`` (no sink; its window and kernels), between two batched
     products per head.  ``up_k`` [H, D, R] and ``up_v`` [H, E, R] are the per-head expansion
-    matrices; ``rotation``: a ``HalfRotation`` over the first entries of the P-part."""
+    matrices; ``rotation``: a ``HalfRotation`` over the first entries of the P-part.  Only c and r
+    are cached, once: the values are read from the key rows (``value_in_key``)."""
 
     def __init__(self, num_heads: int, head_dim: int, rot_dim: int, v_head_dim: int, kv_rank: int,
                  scale: float, window: int, rotation, eps: float):
@@ -237,10 +243,17 @@ class LatentAttention(nn.Module):
         self.eps, self.rotation = eps, rotation
         if rotation.rotary_dim > P:
             raise ValueError("the rotation covers more entries than the rotated part has")
-        self.core = SinkAttention(H, 1, R + P, R, scale, sink=False, window=window)
+        self.core = self.make_core(H, P, R, scale, window)
         self.latent_norm = nn.Parameter(torch.ones(R, dtype=torch.float32), requires_grad=False)
         self.up_k = nn.Parameter(torch.zeros(H, D, R), requires_grad=False)
         self.up_v = nn.Parameter(torch.zeros(H, E, R), requires_grad=False)
+
+    @staticmethod
+    def make_core(num_heads: int, rot_dim: int, kv_rank: int, scale: float, window: int) -> SinkAttention:
+        """A cache holder of this attention (one per pass of a layer that runs several times):
+        one KV head, key rows [c | r], values = the leading R entries of the key rows."""
+        return SinkAttention(num_heads, 1, kv_rank + rot_dim, kv_rank, scale, sink=False,
+                             window=window, value_in_key=True)
 
     def forward(self, q: torch.Tensor, dkv: torch.Tensor, core: Optional[SinkAttention] = None
                 ) -> torch.Tensor:
@@ -254,7 +267,7 @@ class LatentAttention(nn.Module):
         q_abs = torch.bmm(q[:, :, :D].transpose(0, 1), self.up_k)                    # [H, T, R]
         rot = self.rotation
         qf = ops.latent_rope_store(q_abs, q, dkv, self.latent_norm, self.eps, ctx.positions,
-                                   rot.inv_freq, rot.rotary_dim, core.k_cache, core.v_cache,
-                                   ctx.slot_mapping)
+                                   rot.inv_freq, rot.rotary_dim, core.k_cache,
+                                   None if core.value_in_key else core.v_cache, ctx.slot_mapping)
         o = core(qf, None).view(T, H, R)
         return torch.bmm(o.transpose(0, 1), self.up_v.transpose(1, 2)).transpose(0, 1)   # [T, H, E]

@@ -247,8 +247,7 @@ class KidupelLatentMixer(nn.Module):
         rot = HalfRotation(int(m["rot"]["dims"]), float(m["rot"]["base"]))
         self.attn = LatentAttention(H, D, P, E, R, float(m["scale"]), _window(m), rot, eps)
         self.cores = nn.ModuleList([self.attn.core] + [
-            SinkAttention(H, 1, R + P, R, float(m["scale"]), sink=False, window=_window(m))
-            for _ in range(passes - 1)])
+            LatentAttention.make_core(H, P, R, float(m["scale"]), _window(m)) for _ in range(passes - 1)])
         self.sizes = [Q, R + P, H * E]
         self.q_norm = nn.Parameter(torch.ones(Q, dtype=torch.float32), requires_grad=False)
         self.up_q = nn.Parameter(torch.zeros(H * (D + P), Q), requires_grad=False)

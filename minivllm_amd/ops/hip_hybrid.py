@@ -39,14 +39,14 @@ _ghn = _sig("hyb_gated_head_norm", _P, _P, _P, _L, _P, _L, _I, _I, _F, _I, _I, _
 _route = _sig("hyb_grouped_route", _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _P)
 _gelu = _sig("hyb_gelu_route_scale", _P, _P, _P, _L, _I, _I, _I, _P)
 _attn = _sig("hyb_sink_attention_rows", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _I, _P, _P, _L, _P,
-             _F, _L, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P)
+             _F, _L, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P)
 _tiles = _sig("hyb_sink_attention_tiles", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _P, _L, _P, _F,
-              _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P)
+              _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P)
 _tiles_ok = _lib.hyb_sink_attention_tiles_ok
 _tiles_ok.argtypes = [_I, _I]
 _tiles_ok.restype = _I
 _split = _sig("hyb_sink_attention_split", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _L, _P, _P, _F,
-              _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P)
+              _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P)
 _split_ok = _lib.hyb_sink_attention_split_ok
 _split_ok.argtypes = [_I, _I]
 _split_ok.restype = _I
@@ -174,12 +174,25 @@ def _slopes(slopes, H):
     return slopes.data_ptr()
 
 
+def _value_rows(k_cache, v_cache):
+    """Elements from one (slot, KV head) value row to the next.  The V cache is a dense tensor
+    [blocks, block, G, E] or, when the values are stored inside the key rows, a view
+    [blocks, block, G, E] of the leading E entries of each wider row."""
+    n, bs, G, E = v_cache.shape
+    vs = v_cache.stride(2) if G > 1 else v_cache.stride(1)
+    assert v_cache.stride(3) == 1 and vs >= E and v_cache.stride(1) == G * vs \
+        and (n == 1 or v_cache.stride(0) == bs * G * vs), "value rows must be evenly spaced"
+    assert v_cache.dtype == k_cache.dtype and v_cache.shape[:3] == k_cache.shape[:3]
+    return vs
+
+
 def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, scale, sink, gate, out,
                     seq_base=0, window=0, keep_first=0, slopes=None):
     T, H, D = q.shape
     G, E = k_cache.shape[2], v_cache.shape[3]
     assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
-    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype
+    assert k_cache.is_contiguous() and k_cache.dtype == q.dtype
+    vs = _value_rows(k_cache, v_cache)
     assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
     if gate is not None:
         assert gate.stride(1) == 1 and gate.dtype == q.dtype
@@ -188,7 +201,7 @@ def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, s
                  _ptr(_i32(row_seq)), _i32(lens).data_ptr(), len_add,
                  _f32(sink).data_ptr() if sink is not None else None,
                  _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale, T,
-                 H, G, D, E, seq_base, int(window), int(keep_first), _slopes(slopes, H), _dt(q),
+                 H, G, D, E, seq_base, int(window), int(keep_first), _slopes(slopes, H), vs, _dt(q),
                  _stream()), "sink_attention")
     return out
 
@@ -222,7 +235,8 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
     if max_q is None:
         max_q = int((cu_q[1:] - cu_q[:-1]).max())
     assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
-    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype
+    assert k_cache.is_contiguous() and k_cache.dtype == q.dtype
+    vs = _value_rows(k_cache, v_cache)
     assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
     if gate is not None:
         assert gate.stride(1) == 1 and gate.dtype == q.dtype
@@ -231,7 +245,7 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
                   _i32c(cu_q).data_ptr(), _i32(positions).data_ptr(),
                   _f32(sink).data_ptr() if sink is not None else None,
                   _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale,
-                  nseq, 0, max_q, H, G, D, E, int(window), int(keep_first), _slopes(slopes, H),
+                  nseq, 0, max_q, H, G, D, E, int(window), int(keep_first), _slopes(slopes, H), vs,
                   _dt(q), _stream()), "sink_attention_prefill")
     return out
 
@@ -259,9 +273,10 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
     B, H, D = q.shape
     G, E = k_cache.shape[2], v_cache.shape[3]
     es = q.element_size()
+    vs = _value_rows(k_cache, v_cache)
     if (_split_ok(D, E) and q.stride(2) == 1 and q.stride(1) == D and q.data_ptr() % 16 == 0
             and (B == 1 or (q.stride(0) * es) % 16 == 0) and k_cache.is_contiguous()
-            and v_cache.is_contiguous() and out.is_contiguous()):
+            and vs % 8 == 0 and v_cache.data_ptr() % 16 == 0 and out.is_contiguous()):
         seen = max_context_len
         if window and seen:           # what a row can see bounds the useful splits
             seen = min(int(seen), int(window) + int(keep_first))
@@ -275,7 +290,7 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
                       _f32(sink).data_ptr() if sink is not None else None,
                       _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(),
                       ws.data_ptr(), scale, B, H, G, D, E, splits, int(window), int(keep_first),
-                      _slopes(slopes, H), _dt(q), _stream()),
+                      _slopes(slopes, H), vs, _dt(q), _stream()),
                "sink_attention_decode")
         return out
     return _attention_rows(q, k_cache, v_cache, block_tables, None, context_lens, 0, scale, sink,
@@ -545,8 +560,9 @@ def latent_rope_store(q_abs, q, dkv, w, eps, positions, inv_freq, rot_dims, k_ca
     assert q.shape[:2] == (T, H) and q.stride(2) == 1 and q.stride(1) == D + P and dkv.stride(1) == 1
     assert w.numel() == R and inv_freq.numel() * 2 == rot_dims
     if k_cache is not None:
-        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype \
-            and k_cache.shape[2:] == (1, R + P) and v_cache.shape[2:] == (1, R)
+        assert k_cache.is_contiguous() and k_cache.dtype == q.dtype and k_cache.shape[2:] == (1, R + P)
+        if v_cache is not None:          # None: the values are the leading part of the key rows
+            assert v_cache.is_contiguous() and v_cache.shape[2:] == (1, R)
     out = torch.empty((T, H, R + P), dtype=q.dtype, device=q.device)
     _check(_lrs(q_abs.data_ptr(), q.data_ptr(), _rows(q), dkv.data_ptr(), _rows(dkv),
                 _f32(w).data_ptr(), eps, _i32(positions).data_ptr(), _f32(inv_freq).data_ptr(),

@@ -477,7 +477,8 @@ def latent_rope_store(q_abs, q, dkv, w, eps, positions, inv_freq, rot_dims, k_ca
     the heads' unrotated query parts carried into the latent's coordinates; ``q`` [T,H,D+P] whose
     last P entries per head are the part to rotate; ``dkv`` [T,R+P]: the raw latent and one key
     part shared by all heads.  K cache row = [rmsnorm(latent) * w | rotated key part] (one KV
-    head of R + P), V cache row = the normed latent (R).  Returns the queries [T,H,R+P] =
+    head of R + P), V cache row = the normed latent (R; ``v_cache`` None: not written, the reader
+    takes the leading R entries of the key rows).  Returns the queries [T,H,R+P] =
     [q_abs | rotated part].  The rotation turns the first ``rot_dims`` of the P entries."""
     H, T, R = q_abs.shape
     P = dkv.shape[1] - R
@@ -488,7 +489,8 @@ def latent_rope_store(q_abs, q, dkv, w, eps, positions, inv_freq, rot_dims, k_ca
     out = torch.cat([q_abs.transpose(0, 1).float(), qr], -1).to(q.dtype)
     if k_cache is not None and slot_mapping is not None:
         _scatter_rows(k_cache, torch.cat([c, kr], -1)[:, None, :], slot_mapping)
-        _scatter_rows(v_cache, c[:, None, :], slot_mapping)
+        if v_cache is not None:          # None: the values are the leading part of the key rows
+            _scatter_rows(v_cache, c[:, None, :], slot_mapping)
     return out
 
 

@@ -33,9 +33,6 @@ def rms(x, eps):
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
-
 
 def scalar_norm(x, g, eps):
     """RMS norm with a single scalar gain."""

@@ -278,3 +278,42 @@ def test_kernel_state_space_chain(dt, H, G, N, E, taps, parts):
     torch.testing.assert_close(st_g.cpu()[[0, 3]], st_c[[0, 3]], rtol=1e-4, atol=1e-4)
     if taps > 1:
         torch.testing.assert_close(tl_g.cpu()[[0, 3]], tl_c[[0, 3]], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,D,E,window", [(16, 256, 128, 40), (3, 40, 24, 0), (2, 320, 200, 25), (4, 128, 64, 7)])
+def test_kernel_attention_with_values_inside_the_key_rows(dt, H, D, E, window):
+    """One KV head whose value is the leading E entries of its key row (the V cache is a view of
+    the K cache): prompt portions (matrix-core tiles, or rows for sizes without an instance) and
+    decode rows (split contexts, or rows) against the CPU form on the same view."""
+    torch.manual_seed(5)
+    bs, nb = 16, 12
+    kc = (0.5 * torch.randn(nb, bs, 1, D)).to(dt)
+    vc = kc[..., :E]
+    kg = kc.cuda()
+    vg = kg[..., :E]
+    lens_k, lens_q = [70, 33, 5], [70, 9, 5]                 # whole prompt, a late portion, a short one
+    tables = torch.tensor([[3, 1, 7, 9, 11], [0, 2, 4, 0, 0], [5, 0, 0, 0, 0]], dtype=torch.int32)
+    T = sum(lens_q)
+    q = torch.randn(T, H, D).to(dt)
+    cu_q = torch.tensor([0] + list(torch.tensor(lens_q).cumsum(0)), dtype=torch.int32)
+    cu_k = torch.tensor([0] + list(torch.tensor(lens_k).cumsum(0)), dtype=torch.int32)
+    pos = torch.cat([torch.arange(k - n, k) for k, n in zip(lens_k, lens_q)]).to(torch.int32)
+    row_seq = torch.cat([torch.full((n,), i) for i, n in enumerate(lens_q)]).to(torch.int32)
+    scale = D ** -0.5
+    out = torch.zeros(T, H, E, dtype=dt)
+    ref.sink_attention_prefill(q, kc, vc, cu_q, cu_k, tables, scale, None, None, out, window)
+    outg = torch.zeros(T, H, E, dtype=dt, device="cuda")
+    hk.sink_attention_prefill(q.cuda(), kg, vg, cu_q.cuda(), cu_k.cuda(), tables.cuda(), scale, None, None,
+                              outg, positions=pos.cuda(), max_q=max(lens_q), row_seq=row_seq.cuda(),
+                              window=window)
+    torch.testing.assert_close(outg.cpu().float(), out.float(), **tol(dt, 1e-4))
+    qd = torch.randn(3, H, D).to(dt)
+    ctx = torch.tensor(lens_k, dtype=torch.int32)
+    out = torch.zeros(3, H, E, dtype=dt)
+    ref.sink_attention_decode(qd, kc, vc, tables, ctx, scale, None, None, out, window)
+    outg = torch.zeros(3, H, E, dtype=dt, device="cuda")
+    hk.sink_attention_decode(qd.cuda(), kg, vg, tables.cuda(), ctx.cuda(), scale, None, None, outg,
+                             max(lens_k), window=window)
+    torch.testing.assert_close(outg.cpu().float(), out.float(), **tol(dt, 1e-4))
