@@ -159,7 +159,7 @@ def _window(m: dict) -> int:
 
 # ------------------------------------------------------------------ mixers
 # A mixer's ``load`` returns the rows it contributes to the layer's fused projection and their
-# biases (None: none); ``forward(proj, h, out_dtype, which)`` returns [(tensor [T, W], scale)],
+# biases (None: none); ``forward(proj, out_dtype, which)`` returns [(tensor [T, W], scale)],
 # the branches still to be added to the stream; ``which`` is the pass of a looped layer.
 class KidupelParallelMixer(nn.Module):
     def __init__(self, W: int, m: dict, eps: float, passes: int):
@@ -184,7 +184,7 @@ class KidupelParallelMixer(nn.Module):
     def attention_cores(self):
         return list(self.cores)
 
-    def forward(self, proj, h, out_dtype, which):
+    def forward(self, proj, out_dtype, which):
         a = self.cores[which]
         T = proj.shape[0]
         H, G, D, E = a.num_heads, a.num_kv_heads, a.head_dim, a.v_head_dim
@@ -259,7 +259,7 @@ class KidupelLatentMixer(nn.Module):
     def attention_cores(self):
         return list(self.cores)
 
-    def forward(self, proj, h, out_dtype, which):
+    def forward(self, proj, out_dtype, which):
         a = self.attn
         T = proj.shape[0]
         cq, dkv, g = proj[:, :sum(self.sizes)].split(self.sizes, dim=-1)
@@ -309,7 +309,7 @@ class KidupelAttentionMixer(nn.Module):
     def attention_cores(self):
         return list(self.cores)
 
-    def forward(self, proj, h, out_dtype, which):
+    def forward(self, proj, out_dtype, which):
         a = self.cores[which]
         T = proj.shape[0]
         H, G, D, E = a.num_heads, a.num_kv_heads, a.head_dim, a.v_head_dim
@@ -360,7 +360,7 @@ class KidupelLayer(nn.Module):
     def forward(self, h, out_dtype, which: int):
         """h: the layer's normed input.  Returns [(tensor, scale)] still to be added to the stream."""
         proj = F.linear(h, self.in_proj, self.in_bias)
-        ys = self.mix(proj[:, :self.mix_rows], h, out_dtype, which)
+        ys = self.mix(proj[:, :self.mix_rows], out_dtype, which)
         if self.ff:
             ys.append((F.linear(self.act(proj[:, self.mix_rows:self.mix_rows + self.ff], out_dtype), self.down), 1.0))
         return ys
