@@ -110,6 +110,9 @@ class KidupelConfig:
             for a in ([m["left"]] if L.type == "parallel" else [m] if L.type == "attention" else []):
                 if a["heads"] % a.get("kv_heads", a["heads"]):
                     raise ValueError("heads must be a multiple of kv_heads")
+                if int(a.get("vdim", a["dim"])) > 256 or int(a["dim"]) > 1024:
+                    raise ValueError("the attention kernels take keys of at most 1024 and values "
+                                     "of at most 256 numbers per head")
             if L.type == "parallel":
                 r = m["right"]
                 if r["heads"] % r.get("groups", 1) or (r["heads"] * r["vdim"]) % r.get("norm_groups", 1):
