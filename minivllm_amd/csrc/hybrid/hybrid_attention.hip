@@ -48,7 +48,7 @@ struct VisibleKeys {
 
 constexpr int TILE = 256;
 constexpr int RC = 4;       // query heads per workgroup
-constexpr int NACC = 4;     // output columns per thread: RC * E <= NACC * 256
+constexpr int NACC = 4;     // output columns per thread: (heads per workgroup) * E <= NACC * 256
 
 template <typename T>
 __global__ void __launch_bounds__(TILE)
@@ -59,13 +59,15 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
                            int len_add, const float* __restrict__ sink,
                            const T* __restrict__ gate, long gate_row, T* __restrict__ out,
                            float scale, int H, int G, int D, int E, int vec_ok, int seq_base,
-                           KeyRule rule) {
+                           int hpw, KeyRule rule) {
+    // hpw <= RC: query heads per workgroup (fewer when a head's value row is long: the output
+    // columns of a workgroup, hpw * E, are spread over NACC * TILE thread slots)
     extern __shared__ float sm[];
     const int R = H / G;
-    const int chunks = (R + RC - 1) / RC;
+    const int chunks = (R + hpw - 1) / hpw;
     const long t = blockIdx.x;
-    const int g = blockIdx.y / chunks, h0 = g * R + (blockIdx.y % chunks) * RC;
-    const int nr = min(RC, g * R + R - h0);
+    const int g = blockIdx.y / chunks, h0 = g * R + (blockIdx.y % chunks) * hpw;
+    const int nr = min(hpw, g * R + R - h0);
     const int b = row_seq ? row_seq[t] - seq_base : (int)t;      // seq_base: first table row
     if (b < 0) return;
     const int ctx = lens[row_seq ? t : b] + len_add;
@@ -685,8 +687,10 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
     const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E};
     if (rows <= 0) return 0;
     if (rule.v_stride < E) return 1;
-    if (G <= 0 || H % G || RC * E > NACC * TILE || D > 1024) return 1;
-    const int R = H / G, chunks = (R + RC - 1) / RC;
+    if (G <= 0 || H % G || E > NACC * TILE || D > 1024) return 1;
+    const int fit = NACC * TILE / E;                     // heads whose output columns fit
+    const int hpw = fit < RC ? fit : RC;
+    const int R = H / G, chunks = (R + hpw - 1) / hpw;
     const size_t lds = (RC * D + RC * TILE + 4 * RC + 3 * RC + 2) * sizeof(float) + TILE * sizeof(long);
     const int esize = dt == 0 ? 2 : 4;
     const int vec_ok = (D % 4 == 0) && (((size_t)k_cache) % 16 == 0) && ((D * esize) % (4 * esize) == 0);
@@ -696,7 +700,7 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
                                         (const int*)block_tables, max_blocks, block_size,
                                         (const int*)row_seq, (const int*)lens, len_add,
                                         (const float*)sink, (const T*)gate, gate_row, (T*)out,
-                                        scale, H, G, D, E, vec_ok, seq_base, rule));
+                                        scale, H, G, D, E, vec_ok, seq_base, hpw, rule));
     return HYB_LAUNCH_OK();
 }
 

@@ -110,9 +110,9 @@ class KidupelConfig:
             for a in ([m["left"]] if L.type == "parallel" else [m] if L.type == "attention" else []):
                 if a["heads"] % a.get("kv_heads", a["heads"]):
                     raise ValueError("heads must be a multiple of kv_heads")
-                if int(a.get("vdim", a["dim"])) > 256 or int(a["dim"]) > 1024:
-                    raise ValueError("the attention kernels take keys of at most 1024 and values "
-                                     "of at most 256 numbers per head")
+                if int(a.get("vdim", a["dim"])) > 1024 or int(a["dim"]) > 1024:
+                    raise ValueError("the attention kernels take keys and values of at most 1024 "
+                                     "numbers per head")
             if L.type == "parallel":
                 r = m["right"]
                 if r["heads"] % r.get("groups", 1) or (r["heads"] * r["vdim"]) % r.get("norm_groups", 1):
@@ -123,9 +123,9 @@ class KidupelConfig:
             if L.type == "latent_attention":
                 if int(m["rot"]["dims"]) > int(m["rot_dim"]) or int(m["rot"]["dims"]) % 2:
                     raise ValueError("rot.dims must be even and at most rot_dim")
-                if int(m["kv_rank"]) > 256:
-                    raise ValueError("attention over the latent runs with value rows of at most "
-                                     "256 numbers (kv_rank)")
+                if int(m["kv_rank"]) + int(m["rot_dim"]) > 1024:
+                    raise ValueError("attention over the latent runs with key rows of at most "
+                                     "1024 numbers (kv_rank + rot_dim)")
 
 
 def _param(t: torch.Tensor, like: torch.Tensor, dtype=None) -> nn.Parameter:

@@ -92,6 +92,8 @@ ALONE = {
                                                 norm_groups=8), None)], None),
     "latent": ([(fx.latent(), None)], None),
     "latent-partly-rotated": ([(fx.latent(rot_dim=12, rot_dims=8, q_rank=7, kv_rank=24), None)], None),
+    "latent-wide": ([(fx.latent(heads=5, dim=8, rot_dim=6, vdim=8, kv_rank=300, q_rank=9), None)], None),
+    "attention-wide-values": ([(fx.attention(heads=6, kv_heads=2, dim=8, vdim=272, size=5), None)], None),
     "feed-forward": ([(fx.attention(heads=1, kv_heads=1, dim=8, vdim=8), fx.dense())], None),
     "one-layer-three-times": ([(fx.parallel(), fx.dense(16))], (0, 1, 3)),
 }

@@ -282,7 +282,8 @@ def test_kernel_state_space_chain(dt, H, G, N, E, taps, parts):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("H,D,E,window", [(16, 256, 128, 40), (3, 40, 24, 0), (2, 320, 200, 25), (4, 128, 64, 7)])
+@pytest.mark.parametrize("H,D,E,window", [(16, 256, 128, 40), (3, 40, 24, 0), (2, 320, 200, 25), (4, 128, 64, 7),
+                                              (5, 640, 520, 0), (3, 400, 300, 30)])
 def test_kernel_attention_with_values_inside_the_key_rows(dt, H, D, E, window):
     """One KV head whose value is the leading E entries of its key row (the V cache is a view of
     the K cache): prompt portions (matrix-core tiles, or rows for sizes without an instance) and
