@@ -519,6 +519,8 @@ class ModelRunner:
         self.graph_pool = None
         for attn in self._attention_modules():
             attn.k_cache = attn.v_cache = None
+            for attr, _, _ in (self._block_cache_spec(attn) if self.hybrid else []):
+                setattr(attn, attr, None)
         if self.hybrid:
             for d in self.model.state_layers():
                 for attr, _ in d.state_spec():
@@ -601,7 +603,9 @@ class ModelRunner:
         m = self.cfg.model
         itemsize = torch.empty((), dtype=self.kv_dtype).element_size()
         if self.hybrid:
-            return max(1, sum(self.block_size * a.num_kv_heads * itemsize
+            extra = sum(int(np.prod(shape)) * itemsize for a in self.model.attention_layers()
+                        for _, _, shape in self._block_cache_spec(a))
+            return max(1, extra + sum(self.block_size * a.num_kv_heads * itemsize
                               * (a.head_dim + (0 if getattr(a, "value_in_key", False) else a.v_head_dim))
                               for a in self.model.attention_layers()))
         return (2 * m.num_layers * self.block_size * (m.num_kv_heads // self.tp)
@@ -660,20 +664,49 @@ class ModelRunner:
         widest = max([p.shape[0] for p in self.model.parameters() if p.dim() == 2] + [1])
         return 4 * (self.cfg.model.hidden_size * 4 + widest * 3)
 
+    def _block_cache_spec(self, a):
+        f = getattr(a, "block_cache_spec", None)
+        return f(self.block_size) if f else []
+
+    def _paged(self, n: int, rows: int, heads: int, dim: int, behind):
+        """A cache [n, rows, heads, dim] and, for every (rows', heads, dim) of ``behind``, one
+        more [n, rows', heads, dim] directly behind it in the SAME allocation (rows of that width
+        number on from the cache's last row), so kernels address both from one base pointer."""
+        total = n * (rows + sum(r for r, _, _ in behind))
+        flat = torch.zeros(total, heads, dim, dtype=self.kv_dtype, device=self.device)
+        views, at = [flat[:n * rows].view(n, rows, heads, dim)], n * rows
+        for r, h, d in behind:
+            assert (h, d) == (heads, dim), "a cache placed behind another shares its row shape"
+            views.append(flat[at:at + n * r].view(n, r, heads, dim))
+            at += n * r
+        return views
+
     def _allocate_hybrid_caches(self) -> None:
         """One K and one V allocation per attention layer (their head sizes may differ from
         layer to layer and between K and V; a layer whose values are part of its key rows gets a
-        view instead of a V allocation), logical [block, token, kv head, d]; per recurrent
+        view instead of a V allocation), logical [block, token, kv head, d]; whatever further
+        per-page rows a layer's ``block_cache_spec`` lists (pooled keys and values) directly
+        behind the cache they follow; per recurrent
         layer one fp32 row per state slot of whatever the layer's ``state_spec`` lists (matrix
         state, normaliser, running maximum, convolution tail, ...)."""
         n, bs = self.num_kv_blocks, self.block_size
         self.kv_cache = []
         for a in self.model.attention_layers():
-            a.k_cache = torch.zeros(n, bs, a.num_kv_heads, a.head_dim, dtype=self.kv_dtype, device=self.device)
+            spec = self._block_cache_spec(a)
+            kx = [(attr, shape) for attr, after, shape in spec if after == "k_cache"]
+            vx = [(attr, shape) for attr, after, shape in spec if after == "v_cache"]
+            views = self._paged(n, bs, a.num_kv_heads, a.head_dim, [s for _, s in kx])
+            a.k_cache = views[0]
+            for (attr, _), v in zip(kx, views[1:]):
+                setattr(a, attr, v)
             if getattr(a, "value_in_key", False):      # values = leading entries of the key rows
+                assert not vx
                 a.v_cache = a.k_cache[..., :a.v_head_dim]
             else:
-                a.v_cache = torch.zeros(n, bs, a.num_kv_heads, a.v_head_dim, dtype=self.kv_dtype, device=self.device)
+                views = self._paged(n, bs, a.num_kv_heads, a.v_head_dim, [s for _, s in vx])
+                a.v_cache = views[0]
+                for (attr, _), v in zip(vx, views[1:]):
+                    setattr(a, attr, v)
             self.kv_cache.append((a.k_cache, a.v_cache))
         for d in self.model.state_layers():
             for attr, shape in d.state_spec():

@@ -172,12 +172,28 @@ class SinkAttention(nn.Module):
     j < keep_first (the first tokens stay visible at their true positions); ``distance_slopes``
     [H] - slope_h * (i - j) is taken off the score of key j; ``value_in_key`` - a token's value is
     the leading ``v_head_dim`` entries of its key row, so the engine allocates no V cache and
-    ``v_cache`` is a view into ``k_cache``."""
+    ``v_cache`` is a view into ``k_cache``; ``head_temps`` - a learned multiplier per query head
+    on the scaled score (``temps`` [H] fp32); ``softcap`` > 0 - score <- softcap tanh(score /
+    softcap) after scale and temperature; ``pool`` > 0 (needs a window) - besides the window's
+    tokens a query at position i sees ONE key and value for every block of ``pool`` tokens that
+    has passed out of its window as a whole (b pool + pool - 1 <= i - window): the means of the block's
+    cached keys and values, kept in ``k_pool`` / ``v_pool`` [pages, rows, G, D|E] that the engine
+    allocates next to the token caches (``block_cache_spec``) and ``update_pools`` fills once the
+    step's tokens are cached; block rows and token rows are weighed in the same softmax."""
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
                  scale: float, sink: bool = True, window: int = 0, keep_first: int = 0,
-                 distance_slopes: Optional[torch.Tensor] = None, value_in_key: bool = False):
+                 distance_slopes: Optional[torch.Tensor] = None, value_in_key: bool = False,
+                 head_temps: bool = False, softcap: float = 0.0, pool: int = 0):
         super().__init__()
+        if pool and (not window or keep_first or value_in_key or distance_slopes is not None):
+            raise ValueError("pooled blocks need a window and combine with neither kept first "
+                             "tokens, a distance penalty nor values inside the key rows")
+        self.softcap, self.pool = float(softcap), int(pool) if window else 0
+        self.temps = (nn.Parameter(torch.ones(num_heads, dtype=torch.float32), requires_grad=False)
+                      if head_temps else None)
+        self.k_pool: Optional[torch.Tensor] = None
+        self.v_pool: Optional[torch.Tensor] = None
         if value_in_key and v_head_dim > head_dim:
             raise ValueError("values inside the key rows cannot be longer than the keys")
         self.value_in_key = bool(value_in_key)
@@ -193,6 +209,27 @@ class SinkAttention(nn.Module):
         self.k_cache: Optional[torch.Tensor] = None
         self.v_cache: Optional[torch.Tensor] = None
 
+    def block_cache_spec(self, block_size: int):
+        """Further per-page allocations next to the K / V caches: [(attribute, which cache it
+        follows in memory, (rows per page, G, d))].  A pooled row's address is its page's, so
+        rows * pool covers a page of tokens; the engine places each behind the cache named, in
+        ONE allocation, and the kernels reach pooled rows as further rows of that cache."""
+        if not self.pool:
+            return []
+        rows = -(-block_size // self.pool)
+        return [("k_pool", "k_cache", (rows, self.num_kv_heads, self.head_dim)),
+                ("v_pool", "v_cache", (rows, self.num_kv_heads, self.v_head_dim))]
+
+    def update_pools(self) -> None:
+        """After the step's keys and values are cached: the block means of every block that a
+        token of this step completes."""
+        if not self.pool:
+            return
+        ctx = get_context()
+        ops.pool_block_means(self.k_cache, self.v_cache, self.k_pool, self.v_pool, self.pool,
+                             ctx.positions, ctx.block_tables,
+                             ctx.row_seq if ctx.is_prefill else None)
+
     def forward(self, q: torch.Tensor, gate: Optional[torch.Tensor]) -> torch.Tensor:
         """q [T,H,D] (rotated; rows may be strided), gate [T,H] raw or None; K/V of every token
         of the step are in the cache already.  Returns [T, H*E]."""
@@ -203,6 +240,9 @@ class SinkAttention(nn.Module):
         out = torch.zeros((T, self.num_heads, self.v_head_dim), dtype=q.dtype, device=q.device)
         a = (self.k_cache, self.v_cache)
         opt = dict(window=self.window, keep_first=self.keep_first, slopes=self.slopes)
+        if self.temps is not None or self.softcap or self.pool:
+            opt.update(temps=self.temps, softcap=self.softcap, pool=self.pool, k_pool=self.k_pool,
+                       v_pool=self.v_pool)
         if not ctx.is_prefill:
             ops.sink_attention_decode(q, *a, ctx.block_tables, ctx.context_lens, self.scale,
                                       self.sink, gate, out, ctx.max_context_len or None, **opt)

@@ -81,3 +81,42 @@ class RoutedGatedExperts(nn.Module):
             gu = F.linear(h, self.gate_up)
         act = ops.swiglu_route_scale(gu, route, self.ff, self.shared_ff, h.dtype)
         return F.linear(act, self.down)
+
+
+class CappedRoutedExperts(nn.Module):
+    """Gated experts with clamped pre-activations behind a router that renormalises over what it
+    chose, plus an optional shared expert with a per-token gate.
+
+    Router: z = W_r h + b in fp32; the ``top`` largest logits are chosen (ties to the lower
+    index) and their weights are the softmax over those logits alone.  Expert: g = min(gate h, L),
+    u = clamp(up h, -L, L), down(g sigmoid(``slope`` g) (u + 1)), no biases; the routing weight
+    scales the expert's OUTPUT (the down projection is linear, so it is applied to the
+    activation).  Shared expert: the same form with its own size and limit, for every token,
+    times sigmoid(w_s . h); w_s is one more row of the router matrix, so its logit comes out of
+    the same fp32 pass (``ops.grouped_route(..., gates=1)``).
+
+    Execution as for the other routed layers here: one stacked gate+up weight [2 C, W], C =
+    experts * ff + shared_ff (all gate rows, then all up rows), one stacked down weight [W, C],
+    the activation exactly zero for experts a token did not choose: two dense GEMMs and one
+    elementwise kernel, no permutation, no host synchronisation."""
+
+    def __init__(self, hidden_size: int, ff: int, experts: int, top: int, limit: float,
+                 shared_ff: int = 0, shared_limit: float = 0.0, shared_gate: bool = True):
+        super().__init__()
+        if not 0 < top <= experts:
+            raise ValueError("router: `top` must lie in 1 .. experts")
+        self.ff, self.experts, self.top, self.shared_ff = ff, experts, top, shared_ff
+        self.limit, self.shared_limit = float(limit), float(shared_limit)
+        self.gates = 1 if (shared_ff and shared_gate) else 0
+        self.columns = experts * ff + shared_ff
+        f32 = dict(dtype=torch.float32)
+        self.router = nn.Parameter(torch.zeros(experts + self.gates, hidden_size, **f32), requires_grad=False)
+        self.router_bias = nn.Parameter(torch.zeros(experts + self.gates, **f32), requires_grad=False)
+        self.gate_up = nn.Parameter(torch.zeros(2 * self.columns, hidden_size), requires_grad=False)
+        self.down = nn.Parameter(torch.zeros(hidden_size, self.columns), requires_grad=False)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        route = ops.grouped_route(h, self.router, self.top, 1, 1, "chosen", self.router_bias, self.gates)
+        act = ops.capped_glu_route_scale(F.linear(h, self.gate_up), route, self.ff, self.shared_ff,
+                                         self.limit, self.shared_limit, h.dtype)
+        return F.linear(act, self.down)

@@ -104,3 +104,13 @@ def _ensure_builtin() -> None:
         return KidupelForCausalLM
 
     register(["kidupel"], kidupel_cfg, kidupel_class)
+
+    def zegelix_cfg(c, name):
+        from minivllm_amd.models.zegelix import ZegelixConfig
+        return ZegelixConfig.from_dict(c, name)
+
+    def zegelix_class():
+        from minivllm_amd.models.zegelix import ZegelixForCausalLM
+        return ZegelixForCausalLM
+
+    register(["zegelix"], zegelix_cfg, zegelix_class)

@@ -245,8 +245,8 @@ def _seqmix(t):
     return _hybrid() if _on_gpu(t) else torch_seqmix
 
 
-def embed_sum(ids, aux_rows, table, aux_table):
-    return _seqmix(table).embed_sum(ids, aux_rows, table, aux_table)
+def embed_sum(ids, aux_rows, table, aux_table, scale=1.0):
+    return _seqmix(table).embed_sum(ids, aux_rows, table, aux_table, scale)
 
 
 def offset_rms_norm(x, w, eps, out_dtype):
@@ -265,8 +265,12 @@ def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_m
 
 def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
                            positions=None, max_q=None, row_seq=None, first_seq=0,
-                           window=0, keep_first=0, slopes=None):
-    """``positions`` [T], ``max_q`` (longest portion, a host integer), ``row_seq`` and ``first_seq``
+                           window=0, keep_first=0, slopes=None, temps=None, softcap=0.0, pool=0,
+                           k_pool=None, v_pool=None):
+    """``temps`` [H] fp32: a score multiplier per head; ``softcap`` > 0: score <- softcap
+    tanh(score / softcap); ``pool`` > 0 with ``k_pool`` / ``v_pool``: one pooled key / value per
+    block of ``pool`` tokens that has passed out of the window as a whole (``ops.pool_block_means``).
+    ``positions`` [T], ``max_q`` (longest portion, a host integer), ``row_seq`` and ``first_seq``
     (how many sequences of the step precede ``cu_q[0]``'s, i.e. what was sliced off): what the
     GPU kernels take besides (``hip_hybrid.sink_attention_prefill``); the CPU form derives
     everything from ``cu_q`` / ``cu_k``.  ``sink`` None: no sink term.  ``window`` > 0: a query at
@@ -276,9 +280,12 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
         return _hybrid().sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
                                                 scale, sink, gate, out, positions=positions,
                                                 max_q=max_q, row_seq=row_seq, first_seq=first_seq,
-                                                window=window, keep_first=keep_first, slopes=slopes)
+                                                window=window, keep_first=keep_first, slopes=slopes,
+                                                temps=temps, softcap=softcap, pool=pool,
+                                                k_pool=k_pool, v_pool=v_pool)
     return torch_seqmix.sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
-                                               scale, sink, gate, out, window, keep_first, slopes)
+                                               scale, sink, gate, out, window, keep_first, slopes,
+                                               temps, softcap, pool, k_pool, v_pool)
 
 
 def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate,
@@ -290,15 +297,19 @@ def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, s
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
-                          max_context_len=None, window=0, keep_first=0, slopes=None):
+                          max_context_len=None, window=0, keep_first=0, slopes=None, temps=None,
+                          softcap=0.0, pool=0, k_pool=None, v_pool=None):
     """``max_context_len`` (a host integer, an upper bound will do): lets the GPU form size its
     context splits without reading the lengths back."""
     if _on_gpu(q):
         return _hybrid().sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
                                                scale, sink, gate, out, max_context_len,
-                                               window=window, keep_first=keep_first, slopes=slopes)
+                                               window=window, keep_first=keep_first, slopes=slopes,
+                                               temps=temps, softcap=softcap, pool=pool,
+                                               k_pool=k_pool, v_pool=v_pool)
     return torch_seqmix.sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
-                                              scale, sink, gate, out, window, keep_first, slopes)
+                                              scale, sink, gate, out, window, keep_first, slopes,
+                                              temps, softcap, pool, k_pool, v_pool)
 
 
 def unit_norm_store(q, k, eps, k_cache, v_cache, slot_mapping):
@@ -327,8 +338,8 @@ def gated_head_norm(o, w, gate, eps, out_dtype, act="silu"):
     return _seqmix(o).gated_head_norm(o, w, gate, eps, out_dtype, act)
 
 
-def grouped_route(h, router_w, top, groups, keep, score="softmax"):
-    return _seqmix(h).grouped_route(h, router_w, top, groups, keep, score)
+def grouped_route(h, router_w, top, groups, keep, score="softmax", bias=None, gates=0):
+    return _seqmix(h).grouped_route(h, router_w, top, groups, keep, score, bias, gates)
 
 
 def swiglu_route_scale(gu, dense, ff, shared_ff, out_dtype):
@@ -398,3 +409,36 @@ def gated_group_norm(o, skip_x, skip_w, z, w, groups, eps, out_dtype):
 
 def sigmoid_gate(o, gate, out_dtype):
     return _seqmix(o).sigmoid_gate(o, gate, out_dtype)
+
+
+# ---- rotated values, pooled blocks behind a window, real-gated diagonal recurrence, capped experts
+def half_rope_store(q, k, v, positions, inv_freq, rot_dims, v_inv_freq, k_cache, v_cache,
+                    slot_mapping):
+    return _seqmix(q).half_rope_store(q, k, v, positions, inv_freq, rot_dims, v_inv_freq, k_cache,
+                                      v_cache, slot_mapping)
+
+
+def pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions, block_tables, row_seq):
+    return _seqmix(k_cache).pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions,
+                                             block_tables, row_seq)
+
+
+def unturn_gate(o, positions, v_inv_freq, gate, out_dtype):
+    return _seqmix(o).unturn_gate(o, positions, v_inv_freq, gate, out_dtype)
+
+
+def short_conv(x, w, bias, conv_state, cu_q, positions, slots, row_seq=None):
+    """``row_seq`` [T] (GPU, prefill-form steps): the sequence of each row; the CPU form walks
+    ``cu_q``."""
+    if _on_gpu(x):
+        return _hybrid().short_conv(x, w, bias, conv_state, cu_q, positions, slots, row_seq)
+    return torch_seqmix.short_conv(x, w, bias, conv_state, cu_q, positions, slots)
+
+
+def rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp, out_dtype):
+    return _seqmix(u).rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp,
+                                 out_dtype)
+
+
+def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype):
+    return _seqmix(gu).capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype)

@@ -32,12 +32,12 @@ def _bounds(cu_q, positions, B):
 
 
 # ------------------------------------------------------------------ embedding + norms
-def embed_sum(ids, aux_rows, table, aux_table):
-    """fp32 rows ``table[ids] + aux_table[aux_rows]`` (``aux_table`` None: the first alone)."""
+def embed_sum(ids, aux_rows, table, aux_table, scale=1.0):
+    """fp32 rows ``(table[ids] + aux_table[aux_rows]) * scale`` (``aux_table`` None: the first alone)."""
     x = table[ids.long()].float()
     if aux_table is not None:
         x = x + aux_table[aux_rows.long()].float()
-    return x
+    return x * scale if scale != 1.0 else x
 
 
 def offset_rms_norm(x, w, eps, out_dtype):
@@ -111,11 +111,16 @@ def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_m
 
 
 # ------------------------------------------------------------------ attention with a sink
-def _sink_attend(q, k, v, scale, sink, gate, offset, window=0, keep_first=0, slopes=None):
+def _sink_attend(q, k, v, scale, sink, gate, offset, window=0, keep_first=0, slopes=None,
+                 temps=None, softcap=0.0, pool=0, kp=None, vp=None):
     """q [Lq,H,D], k [Lk,G,D], v [Lk,G,E], gate [Lq,H] -> [Lq,H,E] fp32.  Query row i sits at
     position ``offset + i`` and sees key j <= its position; with ``window`` > 0 only keys with
     position - j < window or j < keep_first.  ``slopes`` [H]: slope_h * (position - j) is taken
-    off the score.  ``sink`` None: an ordinary softmax."""
+    off the score.  ``sink`` None: an ordinary softmax.  ``temps`` [H]: the score of head h is
+    multiplied by temps[h]; ``softcap`` > 0: score <- softcap tanh(score / softcap), after scale
+    and temperature.  ``pool`` > 0 (with a window): ``kp`` [Nb,G,D] / ``vp`` [Nb,G,E] hold one key
+    and value per block of ``pool`` tokens; block b joins the softmax of a query at position i
+    when b pool + pool - 1 <= i - window."""
     Lq, H, _ = q.shape
     Lk, G, _ = k.shape
     r = H // G
@@ -131,18 +136,42 @@ def _sink_attend(q, k, v, scale, sink, gate, offset, window=0, keep_first=0, slo
     hidden = kj > qi
     if window:
         hidden = hidden | ((qi - kj >= window) & (kj >= keep_first))
+    hidden = hidden.expand(Lq, Lk)
+    if pool and window and kp is not None and kp.shape[0]:
+        Nb = kp.shape[0]
+        s = torch.cat([s, torch.matmul(qf, kp.float().transpose(0, 1).repeat_interleave(r, 0)
+                                       .transpose(1, 2)) * scale], -1)
+        vf = torch.cat([vf, vp.float().transpose(0, 1).repeat_interleave(r, 0)], 1)
+        last = torch.arange(Nb)[None, :] * pool + pool - 1
+        hidden = torch.cat([hidden, last > qi - window], -1)
+    if temps is not None:
+        s = s * temps.float()[:, None, None]
+    if softcap:
+        s = softcap * torch.tanh(s / softcap)
     s = s.masked_fill(hidden[None], float("-inf"))
+    n_keys = s.shape[-1]
     if sink is not None:
         s = torch.cat([s, sink.float()[:, None, None].expand(H, Lq, 1)], -1)
-    p = torch.softmax(s, -1)[..., :Lk]
+    p = torch.softmax(s, -1)[..., :n_keys]
     o = torch.matmul(p, vf).transpose(0, 1)                           # [Lq, H, E]
     if gate is not None:
         o = o * torch.sigmoid(gate.float())[:, :, None]
     return o
 
 
+def _pooled(k_pool, v_pool, table, ctx, window, pool):
+    """The pooled rows a sequence with ``ctx`` keys can see at its last position."""
+    if not pool or not window or k_pool is None:
+        return None, None
+    nb = max(0, (ctx - window) // pool)
+    if nb == 0:
+        return None, None
+    return _gather_paged(k_pool, table, nb), _gather_paged(v_pool, table, nb)
+
+
 def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
-                           window=0, keep_first=0, slopes=None):
+                           window=0, keep_first=0, slopes=None, temps=None, softcap=0.0, pool=0,
+                           k_pool=None, v_pool=None):
     cq, ck = cu_q.tolist(), cu_k.tolist()
     for b in range(len(cq) - 1):
         s, e = cq[b], cq[b + 1]
@@ -151,21 +180,25 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
             continue
         k = _gather_paged(k_cache, block_tables[b], lk)
         v = _gather_paged(v_cache, block_tables[b], lk)
+        kp, vp = _pooled(k_pool, v_pool, block_tables[b], lk, window, pool)
         out[s:e] = _sink_attend(q[s:e], k, v, scale, sink, None if gate is None else gate[s:e],
-                                lk - (e - s), window, keep_first, slopes).to(out.dtype)
+                                lk - (e - s), window, keep_first, slopes, temps, softcap, pool,
+                                kp, vp).to(out.dtype)
     return out
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
-                          window=0, keep_first=0, slopes=None):
+                          window=0, keep_first=0, slopes=None, temps=None, softcap=0.0, pool=0,
+                          k_pool=None, v_pool=None):
     for b, L in enumerate(context_lens.tolist()):
         if L <= 0:
             continue
         k = _gather_paged(k_cache, block_tables[b], L)
         v = _gather_paged(v_cache, block_tables[b], L)
+        kp, vp = _pooled(k_pool, v_pool, block_tables[b], L, window, pool)
         out[b:b + 1] = _sink_attend(q[b:b + 1], k, v, scale, sink,
                                     None if gate is None else gate[b:b + 1], L - 1, window,
-                                    keep_first, slopes).to(out.dtype)
+                                    keep_first, slopes, temps, softcap, pool, kp, vp).to(out.dtype)
     return out
 
 
@@ -271,11 +304,28 @@ def gated_head_norm(o, w, gate, eps, out_dtype, act="silu"):
 
 
 # ------------------------------------------------------------------ grouped expert routing
-def grouped_route(h, router_w, top, groups, keep, score="softmax"):
+def grouped_route(h, router_w, top, groups, keep, score="softmax", bias=None, gates=0):
     """Scores over all experts in fp32 (``score``: "softmax", or "sigmoid" of each logit); only experts of the ``keep`` groups (of ``groups``
     equal runs of neighbours) whose best score is largest are eligible; the ``top`` largest
-    eligible scores, unnormalised, are the weights.  Returns [T, experts] fp32, zero elsewhere."""
+    eligible scores, unnormalised, are the weights.  Returns [T, experts] fp32, zero elsewhere.
+    ``bias`` [rows]: added to the logits.  ``score`` "chosen": the ``top`` largest LOGITS are
+    chosen and their weights are the softmax over those alone (one group).  ``gates``: that many
+    trailing rows of ``router_w`` are not experts but per-token gates: the result has as many
+    trailing columns holding sigmoid(logit)."""
     z = h.float() @ router_w.float().t()
+    if bias is not None:
+        z = z + bias.float()
+    extra = None
+    if gates:
+        extra = torch.sigmoid(z[:, z.shape[1] - gates:])
+        z = z[:, :z.shape[1] - gates]
+    if score == "chosen":
+        assert groups == 1 and keep == 1
+        ids = torch.sort(z, dim=-1, descending=True, stable=True).indices[:, :top]
+        dense = torch.zeros_like(z)
+        dense.scatter_(1, ids, torch.softmax(z.gather(1, ids), -1))
+        return dense if extra is None else torch.cat([dense, extra], 1)
+    assert not gates
     s = torch.softmax(z, -1) if score == "softmax" else torch.sigmoid(z)
     T, E = s.shape
     per = E // groups
@@ -517,3 +567,132 @@ def sigmoid_gate(o, gate, out_dtype):
     """o [T,H,E] (any strides) * sigmoid(gate [T, H*E]) element by element -> contiguous [T, H*E]."""
     T = o.shape[0]
     return (o.float().reshape(T, -1) * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+# ------------------------------------------------------------------ rotated values, pooled blocks
+def half_rope_store(q, k, v, positions, inv_freq, rot_dims, v_inv_freq, k_cache, v_cache,
+                    slot_mapping):
+    """q [T,H,D], k [T,G,D], v [T,G,E] views of a projection output.  The first ``rot_dims``
+    entries of every q and k head are turned in half-split pairs (entry i with entry i +
+    rot_dims/2) by position * inv_freq[i], q in place and k on its way into the cache.  With
+    ``v_inv_freq`` [E/2] the value heads are turned the same way over ALL their entries (entry m
+    with entry m + E/2 by position * v_inv_freq[m]) before they are cached; None: cached as they
+    are.  Rows with slot < 0 store nothing."""
+    q.copy_(_rotate_half(q.float(), positions, inv_freq, rot_dims).to(q.dtype))
+    kr = _rotate_half(k.float(), positions, inv_freq, rot_dims)
+    vf = v.float()
+    if v_inv_freq is not None:
+        vf = _rotate_half(vf, positions, v_inv_freq, v.shape[-1])
+    if k_cache is not None and slot_mapping is not None:
+        _scatter_rows(k_cache, kr, slot_mapping)
+        _scatter_rows(v_cache, vf, slot_mapping)
+
+
+def pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions, block_tables, row_seq):
+    """For every row of the step whose position ends a block of ``pool`` tokens (position + 1 a
+    multiple of ``pool``): the means of that block's ``pool`` cached key rows and value rows
+    (fp32 sums) are written to the pooled caches.  Block b of a sequence lives in row b %
+    rows_per_page of page block_table[b // rows_per_page] of ``k_pool`` / ``v_pool``
+    [pages, rows_per_page, G, D|E], rows_per_page * pool >= the token page size.  ``row_seq`` [T]:
+    the sequence (block table row) of each row, negative for rows of no sequence; None: row t is
+    sequence t."""
+    bs, pr = k_cache.shape[1], k_pool.shape[1]
+    pos = positions.tolist()
+    seq = row_seq.tolist() if row_seq is not None else list(range(len(pos)))
+    for t, p in enumerate(pos[:len(seq)]):
+        b = seq[t]
+        if b < 0 or b >= block_tables.shape[0] or (p + 1) % pool:
+            continue
+        table = block_tables[b]
+        blk = p // pool
+        js = torch.arange(blk * pool, blk * pool + pool)
+        pages, offs = table[(js // bs)].long(), js % bs
+        page, row = int(table[blk // pr]), blk % pr
+        k_pool[page, row] = k_cache[pages, offs].float().mean(0).to(k_pool.dtype)
+        v_pool[page, row] = v_cache[pages, offs].float().mean(0).to(v_pool.dtype)
+
+
+def unturn_gate(o, positions, v_inv_freq, gate, out_dtype):
+    """o [T,H,E]: every head turned back by its row's position (half-split pairs over all E
+    entries, angles -position * v_inv_freq[m]; None: no turn), then times sigmoid(gate [T, H*E])
+    element by element (None: no gate) -> contiguous [T, H*E]."""
+    T = o.shape[0]
+    of = o.float()
+    if v_inv_freq is not None:
+        of = _rotate_half(of, -positions, v_inv_freq, o.shape[-1])
+    of = of.reshape(T, -1)
+    if gate is not None:
+        of = of * torch.sigmoid(gate.float())
+    return of.to(out_dtype)
+
+
+# ------------------------------------------------------------------ gated diagonal recurrence
+def short_conv(x, w, bias, conv_state, cu_q, positions, slots):
+    """Causal convolution per channel without an activation: x [T, C] (rows may be strided),
+    w [C, taps] fp32 whose LAST column meets the current token, bias [C] or None.  A sequence's
+    last taps-1 inputs live in ``conv_state`` [slots, taps-1, C] fp32 (zeros where it starts at
+    position 0) and are replaced by this step's.  Returns fp32 [T, C]."""
+    xf = x.float()
+    wf = w.float()
+    taps = wf.shape[1]
+    y = torch.zeros_like(xf)
+    for s, e, slot, past in _seq_rows(cu_q, positions, slots):
+        if taps > 1:
+            tail = conv_state[slot] if past else torch.zeros_like(conv_state[slot])
+            full = torch.cat([tail, xf[s:e]], 0)
+            conv_state[slot] = full[full.shape[0] - (taps - 1):]
+        else:
+            full = xf[s:e]
+        y[s:e] = (full.unfold(0, taps, 1) * wf[None]).sum(-1)
+    if bias is not None:
+        y = y + bias.float()
+    return y
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+
+
+def rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp, out_dtype):
+    """Real-gated diagonal recurrence.  u [T, C] fp32; ``gates`` [nb, T, 2c] fp32, C = nb c: for
+    block k of channels the pre-activations of the recurrence gate (first c) and of the input
+    gate (last c), ``gate_bias`` [nb, 2c] still to be added; lam [C];
+        r, i = sigmoid(.);  d = exp(-sharp r softplus(lam));  S <- d S + sqrt(1 - d^2) i u
+    from S = 0 where a sequence starts (``state`` [slots, C] fp32 otherwise, left holding the state
+    after the step).  Returns S * gelu_tanh(y) [T, C] in ``out_dtype`` (y [T, C]: the other
+    branch's pre-activation, rows may be strided)."""
+    T, C = u.shape
+    nb = gates.shape[0]
+    c = C // nb
+    g = torch.sigmoid(gates.float() + gate_bias.float()[:, None, :])          # [nb, T, 2c]
+    r = g[:, :, :c].permute(1, 0, 2).reshape(T, C)
+    i = g[:, :, c:].permute(1, 0, 2).reshape(T, C)
+    d = torch.exp(-sharp * r * F.softplus(lam.float()))
+    add = torch.sqrt(1.0 - d * d) * i * u
+    out = torch.zeros(T, C, dtype=torch.float32)
+    for s, e, slot, past in _seq_rows(cu_q, positions, slots):
+        S = state[slot].clone() if past else torch.zeros(C)
+        for t in range(s, e):
+            S = d[t] * S + add[t]
+            out[t] = S
+        state[slot] = S
+    return (out * gelu_tanh(y.float())).to(out_dtype)
+
+
+def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype):
+    """gu [T, 2 C], C = experts * ff + shared_ff: the gate projections of all experts (and of a
+    shared one behind them), then their up projections.  Column c: g = min(gate, L), u =
+    clamp(up, -L, L), act = w g sigmoid(1.702 g) (u + 1) with L = ``limit`` for routed columns and
+    ``shared_limit`` for shared ones, w = dense[t, expert] for routed columns (exactly zero where w
+    is) and, for shared columns, dense[t, experts] when ``dense`` has that extra column (a
+    per-token gate of the shared expert), else 1.  Returns [T, C]."""
+    T, C = gu.shape[0], gu.shape[1] // 2
+    ne = (C - shared_ff) // ff if ff else 0
+    g, u = gu[:, :C].float(), gu[:, C:2 * C].float()
+    lim = torch.cat([torch.full((ne * ff,), float(limit)), torch.full((shared_ff,), float(shared_limit))])
+    g = torch.minimum(g, lim)
+    u = torch.maximum(torch.minimum(u, lim), -lim)
+    act = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+    sg = dense[:, ne:ne + 1].float() if dense.shape[1] > ne else torch.ones(T, 1)
+    w = torch.cat([dense[:, :ne].float().repeat_interleave(ff, 1), sg.expand(T, shared_ff)], 1)
+    return torch.where(w != 0, act * w, torch.zeros_like(act)).to(out_dtype)
