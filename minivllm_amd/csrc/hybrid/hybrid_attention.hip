@@ -18,7 +18,13 @@
 // maximum then starts at a large negative FINITE number and the sum at 0, so that no path forms
 // inf - inf), a sliding window that keeps the first tokens (a query at position i sees key j <= i
 // only when i - j < window or j < keep_first; keys outside are never loaded), and a distance
-// penalty slope_h * (i - j) taken off the score.
+// penalty slope_h * (i - j) taken off the score; a multiplier per query head on the scaled score
+// (temps), a tanh soft cap (score <- cap tanh(score / cap), after scale and multiplier), and pooled
+// blocks behind the window: with pool = P > 0 a query at position i also sees ONE key / value row
+// for every block b of P tokens with b P + P - 1 <= i - window.  Those rows live in the same
+// allocations as the token rows, pool_base rows behind their start: pooled row b of a sequence is
+// row pool_base + table[b / pool_rows] * pool_rows + b % pool_rows.  In the order the kernels walk
+// a query's keys the pooled rows come first, then the window's tokens.
 #include "hybrid_common.h"
 
 using namespace hyb;
@@ -32,6 +38,24 @@ struct KeyRule {
     int v_stride;           // elements from one (slot, KV head) value row to the next: E for a dense
                             // V cache, more when the value rows are the leading part of wider rows
                             // (values stored inside the key rows: v_cache then points into k_cache)
+    const float* temps;     // [H] or null: multiplies the scaled score of head h
+    float softcap;          // 0: none
+    int pool;               // 0: no pooled blocks (needs window > 0 and keep_first == 0)
+    int pool_rows;          // pooled rows per page
+    long pool_base;         // first pooled row, in rows from the start of the K (and of the V) cache
+    __device__ __forceinline__ float capped(float s) const {
+        return softcap > 0.f ? softcap * tanhf(s / softcap) : s;
+    }
+    __device__ __forceinline__ float head_scale(float scale, int h) const {
+        return temps ? scale * temps[h] : scale;
+    }
+    // pooled blocks a query that sees ctx keys without a window takes in
+    __device__ __forceinline__ int pooled_for(int ctx) const {
+        return (pool > 0 && ctx > window) ? (ctx - window) / pool : 0;
+    }
+    __device__ __forceinline__ long pooled_row(const int* table, int b) const {
+        return pool_base + (long)table[b / pool_rows] * pool_rows + b % pool_rows;
+    }
 };
 
 // The visible keys of a query that sees `ctx` keys without a window (its position is ctx - 1), as
@@ -40,10 +64,16 @@ struct VisibleKeys {
     int kept, lo, count;
     __device__ __forceinline__ VisibleKeys(int ctx, const KeyRule& r) {
         lo = r.window > 0 ? max(0, ctx - r.window) : 0;
-        kept = min(r.keep_first, lo);
+        kept = r.pool > 0 ? r.pooled_for(ctx) : min(r.keep_first, lo);
         count = kept + ctx - lo;
     }
     __device__ __forceinline__ int key(int v) const { return v < kept ? v : lo + (v - kept); }
+    // cache row of virtual key v (with pooled blocks the leading `kept` indices are pooled rows)
+    __device__ __forceinline__ long row(int v, const int* table, int block_size, const KeyRule& r) const {
+        if (r.pool > 0 && v < kept) return r.pooled_row(table, v);
+        const int j = key(v);
+        return (long)table[j / block_size] * block_size + j % block_size;
+    }
 };
 
 constexpr int TILE = 256;
@@ -84,7 +114,7 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
 
     for (int i = tid; i < nr * D; i += TILE) {
         const int r = i / D, d = i - r * D;
-        qs[r * D + d] = ld(q + t * q_row + (long)(h0 + r) * q_head + d) * scale;
+        qs[r * D + d] = ld(q + t * q_row + (long)(h0 + r) * q_head + d) * rule.head_scale(scale, h0 + r);
     }
     if (tid < RC) {
         stat[RC + tid] = tid < nr ? (sink ? sink[h0 + tid] : NO_SINK_MAX) : 0.f;   // running max
@@ -105,7 +135,7 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
 #pragma unroll
         for (int r = 0; r < RC; ++r) s[r] = -INFINITY;
         if (live) {
-            const long slot = (long)table[j / block_size] * block_size + j % block_size;
+            const long slot = vis.row(j0 + tid, table, block_size, rule);
             rowbase[tid] = slot;
             const T* kr = k_cache + (slot * G + g) * (long)D;
 #pragma unroll
@@ -130,7 +160,7 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
             }
             const float dist = (float)(ctx - 1 - j);
 #pragma unroll
-            for (int r = 0; r < RC; ++r) s[r] -= slope[r] * dist;
+            for (int r = 0; r < RC; ++r) s[r] = rule.capped(s[r]) - slope[r] * dist;
         }
         // tile maximum per head
 #pragma unroll
@@ -241,6 +271,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
     const bool qok = qi < qlen;
     const int qpos = start + qi;
 
+    const float hscale = rule.head_scale(scale, h);
     float qreg[QK16 ? 1 : DP / 2];
     bf16x8 qv[QK16 ? DP / 16 : 1];
     {
@@ -261,7 +292,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
 #pragma unroll
             for (int s = 0; s < DP / 2; ++s) {
                 const int d = 2 * s + half;
-                qreg[s] = (qok && d < D) ? ld(qp + d) * scale : 0.f;
+                qreg[s] = (qok && d < D) ? ld(qp + d) * hscale : 0.f;
             }
             for (int i = tid; i < 32 * (KS - D); i += 256) {      // padding columns of K stay zero
                 const int key = i / (KS - D), c = D + i - key * (KS - D);
@@ -284,16 +315,26 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
     const int wg_lo = rule.window > 0 ? max(0, start + tile * 128 - rule.window + 1) : 0;
     const int wave_lo = rule.window > 0 ? max(0, start + tile * 128 + wave * 32 - rule.window + 1) : 0;
 
-    for (int k0 = 0; k0 < wg_ctx; k0 += 32) {
-        if (k0 >= rule.keep_first && k0 + 32 <= wg_lo) continue;     // (uniform) nobody sees this tile
+    // pooled rows first (those the workgroup's last query takes in), then the tokens
+    const int wg_nb = rule.pooled_for(wg_ctx), ptiles = (wg_nb + 31) / 32;
+    const int wave_nb = rule.pooled_for(wave_last + 1), q_nb = rule.pooled_for(qpos + 1);
+    for (int it = 0; it < ptiles + (wg_ctx + 31) / 32; ++it) {
+        const bool pooled = it < ptiles;                              // (uniform)
+        const int k0 = (pooled ? it : it - ptiles) * 32;
+        const int k_lim = pooled ? wg_nb : wg_ctx;
+        if (!pooled && k0 >= rule.keep_first && k0 + 32 <= wg_lo) continue;   // (uniform) nobody sees this tile
+        auto cache_row = [&](int j) -> long {
+            return pooled ? rule.pooled_row(table, j)
+                          : (long)table[j / block_size] * block_size + j % block_size;
+        };
         // ---- K and V tile into LDS
         if constexpr (QK16) {
             const int D8 = D >> 3;
             for (int i = tid; i < 32 * D8; i += 256) {
                 const int key = i / D8, c = (i - key * D8) << 3, j = k0 + key;
                 uint4 raw = make_uint4(0, 0, 0, 0);
-                if (j < wg_ctx) {
-                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                if (j < k_lim) {
+                    const long slot = cache_row(j);
                     raw = *reinterpret_cast<const uint4*>(k_cache + (slot * G + g) * (long)D + c);
                 }
                 *reinterpret_cast<uint4*>(Kb + key * KSB + c) = raw;
@@ -303,8 +344,8 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
             for (int i = tid; i < 32 * D4; i += 256) {
                 const int key = i / D4, c = (i - key * D4) << 2, j = k0 + key;
                 float v4[4] = {0.f, 0.f, 0.f, 0.f};
-                if (j < wg_ctx) {
-                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                if (j < k_lim) {
+                    const long slot = cache_row(j);
                     Vec4<T>::load(k_cache + (slot * G + g) * (long)D + c, v4);
                 }
                 float* dst = Ks + key * KS + c;
@@ -314,8 +355,8 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
             for (int i = tid; i < 32 * D; i += 256) {
                 const int key = i / D, c = i - key * D, j = k0 + key;
                 float v = 0.f;
-                if (j < wg_ctx) {
-                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                if (j < k_lim) {
+                    const long slot = cache_row(j);
                     v = ld(k_cache + (slot * G + g) * (long)D + c);
                 }
                 Ks[key * KS + c] = v;
@@ -326,8 +367,8 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
             for (int i = tid; i < 32 * E4; i += 256) {
                 const int key = i / E4, c = (i - key * E4) << 2, j = k0 + key;
                 float v4[4] = {0.f, 0.f, 0.f, 0.f};
-                if (j < wg_ctx) {
-                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                if (j < k_lim) {
+                    const long slot = cache_row(j);
                     Vec4<T>::load(v_cache + (slot * G + g) * (long)rule.v_stride + c, v4);
                 }
                 float* dst = Vs + key * EP + c;
@@ -337,15 +378,16 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
             for (int i = tid; i < 32 * E; i += 256) {
                 const int key = i / E, c = i - key * E, j = k0 + key;
                 float v = 0.f;
-                if (j < wg_ctx) {
-                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                if (j < k_lim) {
+                    const long slot = cache_row(j);
                     v = ld(v_cache + (slot * G + g) * (long)rule.v_stride + c);
                 }
                 Vs[key * EP + c] = v;
             }
         }
         __syncthreads();
-        if (wave_live && k0 <= wave_last && (k0 < rule.keep_first || k0 + 32 > wave_lo)) {
+        if (wave_live && (pooled ? k0 < wave_nb
+                                 : (k0 <= wave_last && (k0 < rule.keep_first || k0 + 32 > wave_lo)))) {
             f32x16 sacc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
@@ -357,7 +399,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                     sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qv[s], sacc, 0, 0, 0);
                 }
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[r] *= scale;
+                for (int r = 0; r < 16; ++r) sacc[r] *= hscale;
             } else {
                 const float* ka = Ks + l32 * KS + half;
 #pragma unroll
@@ -368,9 +410,9 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                const bool seen = qok && key <= qpos &&
-                                  (rule.window <= 0 || qpos - key < rule.window || key < rule.keep_first);
-                const float v = seen ? sacc[r] - slope * (float)(qpos - key) : -INFINITY;
+                const bool seen = qok && (pooled ? key < q_nb : (key <= qpos &&
+                                  (rule.window <= 0 || qpos - key < rule.window || key < rule.keep_first)));
+                const float v = seen ? rule.capped(sacc[r]) - (pooled ? 0.f : slope * (float)(qpos - key)) : -INFINITY;
                 sacc[r] = v;
                 mt = fmaxf(mt, v);
             }
@@ -477,8 +519,9 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
     for (int r = 0; r < RC; ++r) {
         if (r < nr) {
             load_run<T, EPL>(q + b * q_row + (long)(h0 + r) * q_head + lane16 * EPL, qf[r]);
+            const float hs = rule.head_scale(scale, h0 + r);
 #pragma unroll
-            for (int i = 0; i < EPL; ++i) qf[r][i] *= scale;
+            for (int i = 0; i < EPL; ++i) qf[r][i] *= hs;
             m[r] = sink ? sink[h0 + r] : NO_SINK_MAX;
             slope[r] = rule.slopes ? rule.slopes[h0 + r] : 0.f;
         } else {
@@ -496,8 +539,8 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
         const bool two = vj + 16 < k_end;
         const int j = vis.key(vj), j2 = two ? vis.key(vj + 16) : j;
         const float dist[2] = {(float)(ctx - 1 - j), (float)(ctx - 1 - j2)};
-        const long slot = (long)table[j / block_size] * block_size + j % block_size;
-        const long slot2 = two ? (long)table[j2 / block_size] * block_size + j2 % block_size : slot;
+        const long slot = vis.row(vj, table, block_size, rule);
+        const long slot2 = two ? vis.row(vj + 16, table, block_size, rule) : slot;
         float kf[2][EPL], vf[2][VPL];
         load_run<T, EPL>(k_cache + (slot * G + g) * (long)D + lane16 * EPL, kf[0]);
         load_run<T, EPL>(k_cache + (slot2 * G + g) * (long)D + lane16 * EPL, kf[1]);
@@ -516,7 +559,7 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
                 d += __shfl_xor(d, 2, kWave);
                 d += __shfl_xor(d, 4, kWave);
                 d += __shfl_xor(d, 8, kWave);
-                d -= slope[r] * dist[x];
+                d = rule.capped(d) - slope[r] * dist[x];
                 if (d > m[r]) {                    // the running maximum moves: rescale (rare)
                     const float a = expf(m[r] - d);
                     l[r] *= a;
@@ -602,6 +645,12 @@ static int launch_split(const void* q, long q_row, long q_head, const void* k_ca
     return HYB_LAUNCH_OK();
 }
 
+// pooled blocks need a window, no kept first tokens, no distance penalty, and a place in the caches
+static bool pool_rule_ok(const KeyRule& r) {
+    return r.pool == 0 || (r.pool > 0 && r.window > 0 && r.keep_first == 0 && !r.slopes &&
+                           r.pool_rows > 0 && r.pool_base > 0);
+}
+
 extern "C" {
 
 // 1 when the split decode kernel has an instance for these head sizes
@@ -615,9 +664,13 @@ int hyb_sink_attention_split(const void* q, long q_row, long q_head, const void*
                              int block_size, const void* context_lens, const void* sink,
                              const void* gate, long gate_row, void* out, void* ws, float scale,
                              int B, int H, int G, int D, int E, int splits, int window,
-                             int keep_first, const void* slopes, int v_stride, int dt, hipStream_t s) {
-    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E};
+                             int keep_first, const void* slopes, int v_stride, const void* temps,
+                             float softcap, int pool, int pool_rows, long pool_base, int dt,
+                             hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E,
+                       (const float*)temps, softcap, pool, pool_rows, pool_base};
     if (B <= 0) return 0;
+    if (!pool_rule_ok(rule)) return 1;
     if (G <= 0 || H % G || splits < 1 || !hyb_sink_attention_split_ok(D, E)) return 1;
     if (rule.v_stride < E || rule.v_stride % 8) return 1;      // 16-byte runs of a value row
     if (((size_t)k_cache | (size_t)v_cache | (size_t)q) % 16 || (q_row * (dt == 0 ? 2 : 4)) % 16) return 1;
@@ -650,9 +703,12 @@ int hyb_sink_attention_tiles(const void* q, long q_row, long q_head, const void*
                              const void* sink, const void* gate, long gate_row, void* out,
                              float scale, int nseq, int seq0, int max_q, int H, int G, int D,
                              int E, int window, int keep_first, const void* slopes, int v_stride,
-                             int dt, hipStream_t s) {
-    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E};
+                             const void* temps, float softcap, int pool, int pool_rows,
+                             long pool_base, int dt, hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E,
+                       (const float*)temps, softcap, pool, pool_rows, pool_base};
     if (nseq <= 0 || max_q <= 0) return 0;
+    if (!pool_rule_ok(rule)) return 1;
     if (rule.v_stride < E) return 1;
     if (G <= 0 || H % G || !hyb_sink_attention_tiles_ok(D, E)) return 1;
 #define TILES_ARGS q, q_row, q_head, k_cache, v_cache, block_tables, max_blocks, block_size, cu_q, \
@@ -682,10 +738,13 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
                             int block_size, const void* row_seq, const void* lens, int len_add,
                             const void* sink, const void* gate, long gate_row, void* out,
                             float scale, long rows, int H, int G, int D, int E, int seq_base,
-                            int window, int keep_first, const void* slopes, int v_stride, int dt,
-                            hipStream_t s) {
-    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E};
+                            int window, int keep_first, const void* slopes, int v_stride,
+                            const void* temps, float softcap, int pool, int pool_rows,
+                            long pool_base, int dt, hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes, v_stride > 0 ? v_stride : E,
+                       (const float*)temps, softcap, pool, pool_rows, pool_base};
     if (rows <= 0) return 0;
+    if (!pool_rule_ok(rule)) return 1;
     if (rule.v_stride < E) return 1;
     if (G <= 0 || H % G || E > NACC * TILE || D > 1024) return 1;
     const int fit = NACC * TILE / E;                     // heads whose output columns fit

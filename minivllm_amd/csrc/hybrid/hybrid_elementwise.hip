@@ -5,16 +5,16 @@
 
 using namespace hyb;
 
-// x[t] = table[ids[t]] + aux[aux_rows[t]]  (fp32 out)
+// x[t] = (table[ids[t]] + aux[aux_rows[t]]) * scale  (fp32 out)
 template <typename T>
 __global__ void embed_sum_kernel(const int* __restrict__ ids, const int* __restrict__ aux_rows,
                                  const T* __restrict__ table, const T* __restrict__ aux,
-                                 float* __restrict__ x, int W) {
+                                 float* __restrict__ x, int W, float scale) {
     const long t = blockIdx.x;
     const T* a = table + (long)ids[t] * W;
     const T* b = aux ? aux + (long)aux_rows[t] * W : nullptr;
     for (int c = threadIdx.x; c < W; c += blockDim.x)
-        x[t * W + c] = ld(a + c) + (b ? ld(b + c) : 0.f);
+        x[t * W + c] = (ld(a + c) + (b ? ld(b + c) : 0.f)) * scale;
 }
 
 // out[t] = x[t] / rms(x[t]) * (1 + w)
@@ -241,11 +241,11 @@ static inline int threads_for(int n) { return n >= 1024 ? 512 : n >= 256 ? 256 :
 extern "C" {
 
 int hyb_embed_sum(const void* ids, const void* aux_rows, const void* table, const void* aux,
-                  void* x, long T_, int W, int dt, hipStream_t s) {
+                  void* x, long T_, int W, float scale, int dt, hipStream_t s) {
     if (T_ <= 0) return 0;
     HYB_DISPATCH(dt, hipLaunchKernelGGL(embed_sum_kernel<T>, dim3(T_), dim3(threads_for(W)), 0, s,
                                         (const int*)ids, (const int*)aux_rows, (const T*)table,
-                                        (const T*)aux, (float*)x, W));
+                                        (const T*)aux, (float*)x, W, scale));
     return HYB_LAUNCH_OK();
 }
 

@@ -228,7 +228,7 @@ class SinkAttention(nn.Module):
         ctx = get_context()
         ops.pool_block_means(self.k_cache, self.v_cache, self.k_pool, self.v_pool, self.pool,
                              ctx.positions, ctx.block_tables,
-                             ctx.row_seq if ctx.is_prefill else None)
+                             ctx.row_seq if ctx.is_prefill else None, ctx.slot_mapping)
 
     def forward(self, q: torch.Tensor, gate: Optional[torch.Tensor]) -> torch.Tensor:
         """q [T,H,D] (rotated; rows may be strided), gate [T,H] raw or None; K/V of every token

@@ -418,9 +418,10 @@ def half_rope_store(q, k, v, positions, inv_freq, rot_dims, v_inv_freq, k_cache,
                                       v_cache, slot_mapping)
 
 
-def pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions, block_tables, row_seq):
+def pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions, block_tables, row_seq,
+                     slot_mapping):
     return _seqmix(k_cache).pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions,
-                                             block_tables, row_seq)
+                                             block_tables, row_seq, slot_mapping)
 
 
 def unturn_gate(o, positions, v_inv_freq, gate, out_dtype):

@@ -30,7 +30,7 @@ def _sig(name, *argtypes):
     return f
 
 
-_embed = _sig("hyb_embed_sum", _P, _P, _P, _P, _P, _L, _I, _I, _P)
+_embed = _sig("hyb_embed_sum", _P, _P, _P, _P, _P, _L, _I, _F, _I, _P)
 _norm = _sig("hyb_offset_rms_norm", _P, _P, _P, _L, _I, _F, _I, _P)
 _post = _sig("hyb_post_norm_residual", _P, _L, _P, _P, _P, _P, _L, _I, _F, _I, _P)
 _rope = _sig("hyb_pair_rope_mix_store", _P, _P, _P, _L, _P, _P, _I, _P, _P, _I, _P, _P, _P, _L,
@@ -38,15 +38,16 @@ _rope = _sig("hyb_pair_rope_mix_store", _P, _P, _P, _L, _P, _P, _I, _P, _P, _I, 
 _ghn = _sig("hyb_gated_head_norm", _P, _P, _P, _L, _P, _L, _I, _I, _F, _I, _I, _I, _P)
 _route = _sig("hyb_grouped_route", _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _P)
 _gelu = _sig("hyb_gelu_route_scale", _P, _P, _P, _L, _I, _I, _I, _P)
+_POOL = (_P, _F, _I, _I, _L)        # head temperatures, soft cap, pool, pooled rows per page, first pooled row
 _attn = _sig("hyb_sink_attention_rows", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _I, _P, _P, _L, _P,
-             _F, _L, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P)
+             _F, _L, _I, _I, _I, _I, _I, _I, _I, _P, _I, *_POOL, _I, _P)
 _tiles = _sig("hyb_sink_attention_tiles", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _P, _L, _P, _F,
-              _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P)
+              _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, *_POOL, _I, _P)
 _tiles_ok = _lib.hyb_sink_attention_tiles_ok
 _tiles_ok.argtypes = [_I, _I]
 _tiles_ok.restype = _I
 _split = _sig("hyb_sink_attention_split", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _L, _P, _P, _F,
-              _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P)
+              _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, *_POOL, _I, _P)
 _split_ok = _lib.hyb_sink_attention_split_ok
 _split_ok.argtypes = [_I, _I]
 _split_ok.restype = _I
@@ -72,6 +73,13 @@ _lrs = _sig("hyb_latent_rope_store", _P, _P, _L, _P, _L, _P, _F, _P, _P, _I, _P,
 _xie = _sig("hyb_xielu", _P, _L, _P, _L, _I, _F, _F, _I, _P)
 _ggn = _sig("hyb_gated_group_norm", _P, _P, _P, _P, _L, _P, _P, _L, _I, _I, _I, _F, _I, _P)
 _sgt = _sig("hyb_sigmoid_gate", _P, _L, _L, _P, _L, _P, _L, _I, _I, _I, _P)
+_hrs = _sig("hyb_half_rope_store", _P, _P, _P, _L, _P, _P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P)
+_pbm = _sig("hyb_pool_block_means", _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _I, _I, _I, _I, _I, _I, _I, _P)
+_utg = _sig("hyb_unturn_gate", _P, _L, _L, _P, _P, _P, _L, _P, _L, _I, _I, _I, _P)
+_scv = _sig("hyb_short_conv", _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P)
+_lru = _sig("hyb_rglru_scan", _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _F, _I, _I, _P)
+_crt = _sig("hyb_chosen_route", _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P)
+_cgl = _sig("hyb_capped_glu_route_scale", _P, _L, _P, _P, _L, _I, _I, _I, _I, _F, _F, _I, _P)
 
 _DT = {torch.bfloat16: 0, torch.float32: 2}
 
@@ -116,11 +124,11 @@ def _rows(t: torch.Tensor) -> int:
 
 
 # ------------------------------------------------------------------ embedding + norms
-def embed_sum(ids, aux_rows, table, aux_table):
+def embed_sum(ids, aux_rows, table, aux_table, scale=1.0):
     T, W = ids.shape[0], table.shape[1]
     x = torch.empty((T, W), dtype=torch.float32, device=table.device)
     _check(_embed(_ptr(_i32(ids)), _ptr(_i32(aux_rows)) if aux_table is not None else None,
-                  table.data_ptr(), _ptr(aux_table), x.data_ptr(), T, W, _dt(table), _stream()),
+                  table.data_ptr(), _ptr(aux_table), x.data_ptr(), T, W, float(scale), _dt(table), _stream()),
            "embed_sum")
     return x
 
@@ -186,8 +194,31 @@ def _value_rows(k_cache, v_cache):
     return vs
 
 
+def _pool_args(k_cache, v_cache, vs, H, temps, softcap, pool, k_pool, v_pool):
+    """(temps, softcap, pool, pooled rows per page, first pooled row) for the attention kernels.
+    The pooled caches lie behind the token caches in the same allocations, the same number of
+    rows behind both."""
+    tp = None
+    if temps is not None:
+        assert temps.dtype == torch.float32 and temps.is_contiguous() and temps.numel() == H
+        tp = temps.data_ptr()
+    if not pool:
+        return tp, float(softcap), 0, 0, 0
+    n, bs, G, D = k_cache.shape
+    es = k_cache.element_size()
+    assert k_pool.is_contiguous() and v_pool.is_contiguous() and k_pool.shape[0] == n \
+        and k_pool.shape[2:] == (G, D) and v_pool.shape[:3] == k_pool.shape[:3] \
+        and k_pool.shape[1] * pool >= bs and k_pool.dtype == k_cache.dtype
+    base = (k_pool.data_ptr() - k_cache.data_ptr()) // (G * D * es)
+    assert base > 0 and k_cache.data_ptr() + base * G * D * es == k_pool.data_ptr() \
+        and v_cache.data_ptr() + base * G * vs * es == v_pool.data_ptr(), \
+        "the pooled rows must follow their token cache in one allocation"
+    return tp, float(softcap), int(pool), int(k_pool.shape[1]), int(base)
+
+
 def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, scale, sink, gate, out,
-                    seq_base=0, window=0, keep_first=0, slopes=None):
+                    seq_base=0, window=0, keep_first=0, slopes=None, temps=None, softcap=0.0, pool=0,
+                    k_pool=None, v_pool=None):
     T, H, D = q.shape
     G, E = k_cache.shape[2], v_cache.shape[3]
     assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
@@ -201,23 +232,25 @@ def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, s
                  _ptr(_i32(row_seq)), _i32(lens).data_ptr(), len_add,
                  _f32(sink).data_ptr() if sink is not None else None,
                  _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale, T,
-                 H, G, D, E, seq_base, int(window), int(keep_first), _slopes(slopes, H), vs, _dt(q),
+                 H, G, D, E, seq_base, int(window), int(keep_first), _slopes(slopes, H), vs,
+                 *_pool_args(k_cache, v_cache, vs, H, temps, softcap, pool, k_pool, v_pool), _dt(q),
                  _stream()), "sink_attention")
     return out
 
 
 def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate, out,
-                        seq_base=0, window=0, keep_first=0, slopes=None):
+                        seq_base=0, window=0, keep_first=0, slopes=None, **pooled):
     """Rows of a prefill-form step, one workgroup per row: row t belongs to sequence
     ``row_seq[t]`` (< ``seq_base``: skipped), whose block table is row ``row_seq[t] - seq_base``
     of ``block_tables``, and sees ``positions[t] + 1`` keys."""
     return _attention_rows(q, k_cache, v_cache, block_tables, row_seq, positions, 1, scale, sink,
-                           gate, out, seq_base, window, keep_first, slopes)
+                           gate, out, seq_base, window, keep_first, slopes, **pooled)
 
 
 def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
                            positions=None, max_q=None, row_seq=None, first_seq=0,
-                           window=0, keep_first=0, slopes=None):
+                           window=0, keep_first=0, slopes=None, temps=None, softcap=0.0, pool=0,
+                           k_pool=None, v_pool=None):
     """The prompt portions of a step: sequence b owns rows cu_q[b] .. cu_q[b+1] (absolute rows
     of q / out / positions) and block table row b.  Runs the matrix-core tile kernel (fp32
     scores, weights and sums); head sizes it has no instance for go row by row.  ``cu_k`` is
@@ -231,7 +264,8 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
         # ``first_seq``: number of the step's sequences ahead of these (its decode riders)
         return sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale,
                                    sink, gate, out, seq_base=first_seq, window=window,
-                                   keep_first=keep_first, slopes=slopes)
+                                   keep_first=keep_first, slopes=slopes, temps=temps,
+                                   softcap=softcap, pool=pool, k_pool=k_pool, v_pool=v_pool)
     if max_q is None:
         max_q = int((cu_q[1:] - cu_q[:-1]).max())
     assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
@@ -246,6 +280,7 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
                   _f32(sink).data_ptr() if sink is not None else None,
                   _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale,
                   nseq, 0, max_q, H, G, D, E, int(window), int(keep_first), _slopes(slopes, H), vs,
+                  *_pool_args(k_cache, v_cache, vs, H, temps, softcap, pool, k_pool, v_pool),
                   _dt(q), _stream()), "sink_attention_prefill")
     return out
 
@@ -265,7 +300,8 @@ def decode_splits(batch: int, kv_heads: int, heads: int, max_context_len) -> int
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
-                          max_context_len=None, window=0, keep_first=0, slopes=None):
+                          max_context_len=None, window=0, keep_first=0, slopes=None, temps=None,
+                          softcap=0.0, pool=0, k_pool=None, v_pool=None):
     """Single next tokens: row b is sequence b with ``context_lens[b]`` keys.  Head sizes the
     split-context kernel has an instance for (D in 64 / 128 / 256, E in 64 / 128) stream K / V
     rows with coalesced 16-byte loads over several workgroups per sequence and are merged by a
@@ -279,7 +315,7 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
             and vs % 8 == 0 and v_cache.data_ptr() % 16 == 0 and out.is_contiguous()):
         seen = max_context_len
         if window and seen:           # what a row can see bounds the useful splits
-            seen = min(int(seen), int(window) + int(keep_first))
+            seen = min(int(seen), int(window) + int(keep_first) + (int(seen) // pool if pool else 0))
         splits = decode_splits(B, G, H, seen)
         ws = torch.empty((B * H * splits * (E + 2),), dtype=torch.float32, device=q.device)
         if gate is not None:
@@ -290,11 +326,13 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
                       _f32(sink).data_ptr() if sink is not None else None,
                       _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(),
                       ws.data_ptr(), scale, B, H, G, D, E, splits, int(window), int(keep_first),
-                      _slopes(slopes, H), vs, _dt(q), _stream()),
+                      _slopes(slopes, H), vs,
+                      *_pool_args(k_cache, v_cache, vs, H, temps, softcap, pool, k_pool, v_pool),
+                      _dt(q), _stream()),
                "sink_attention_decode")
         return out
     return _attention_rows(q, k_cache, v_cache, block_tables, None, context_lens, 0, scale, sink,
-                           gate, out, 0, window, keep_first, slopes)
+                           gate, out, 0, window, keep_first, slopes, temps, softcap, pool, k_pool, v_pool)
 
 
 # ------------------------------------------------------------------ gated delta rule
@@ -366,9 +404,16 @@ def gated_head_norm(o, w, gate, eps, out_dtype, act="silu"):
 
 
 # ------------------------------------------------------------------ grouped expert routing
-def grouped_route(h, router_w, top, groups, keep, score="softmax"):
-    assert score in ("softmax", "sigmoid")
+def grouped_route(h, router_w, top, groups, keep, score="softmax", bias=None, gates=0):
     T, W = h.shape
+    if score == "chosen":
+        NR = router_w.shape[0]
+        assert groups == 1 and keep == 1 and h.is_contiguous() and 0 <= gates < NR
+        dense = torch.empty((T, NR), dtype=torch.float32, device=h.device)
+        _check(_crt(h.data_ptr(), _f32(router_w).data_ptr(), _ptr(_f32(bias)) if bias is not None else None,
+                    dense.data_ptr(), T, W, NR - gates, NR, top, _dt(h), _stream()), "chosen_route")
+        return dense
+    assert score in ("softmax", "sigmoid") and bias is None and not gates
     NE = router_w.shape[0]
     assert h.is_contiguous()
     dense = torch.empty((T, NE), dtype=torch.float32, device=h.device)
@@ -599,3 +644,109 @@ def sigmoid_gate(o, gate, out_dtype):
     _check(_sgt(o.data_ptr(), o.stride(0), o.stride(1), gate.data_ptr(), _rows(gate), out.data_ptr(),
                 T, H, E, _dt(o), _stream()), "sigmoid_gate")
     return out
+
+
+# ------------------------------------------------------------------ rotated values, pooled blocks
+def half_rope_store(q, k, v, positions, inv_freq, rot_dims, v_inv_freq, k_cache, v_cache, slot_mapping):
+    T, H, D = q.shape
+    G, E = v.shape[1], v.shape[2]
+    rs = q.stride(0)
+    assert (T == 1 or (k.stride(0) == rs and v.stride(0) == rs)) and q.stride(1) == D \
+        and k.stride(1) == D and v.stride(1) == E and q.stride(2) == 1, \
+        "q / k / v must be views of one projection output"
+    if k_cache is not None:
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype \
+            and k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, E)
+    if rot_dims:
+        assert inv_freq.numel() * 2 == rot_dims
+    if v_inv_freq is not None:
+        assert v_inv_freq.numel() * 2 == E
+    _check(_hrs(q.data_ptr(), k.data_ptr(), v.data_ptr(), rs if T > 1 else int(rs or 0),
+                _i32(positions).data_ptr(), _ptr(_f32(inv_freq)) if rot_dims else None, int(rot_dims),
+                _ptr(_f32(v_inv_freq)) if v_inv_freq is not None else None, _ptr(k_cache), _ptr(v_cache),
+                _ptr(_i32(slot_mapping)), T, H, G, D, E, _dt(q), _stream()), "half_rope_store")
+
+
+def pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions, block_tables, row_seq,
+                     slot_mapping):
+    n, bs, G, D = k_cache.shape
+    E = v_cache.shape[3]
+    T = positions.shape[0] if row_seq is None else min(positions.shape[0], row_seq.shape[0])
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_pool.is_contiguous() \
+        and v_pool.is_contiguous() and k_pool.dtype == k_cache.dtype and v_pool.dtype == k_cache.dtype
+    assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
+    if row_seq is None:
+        assert block_tables.shape[0] >= T
+    _check(_pbm(k_cache.data_ptr(), v_cache.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
+                _i32(positions).data_ptr(), _i32(slot_mapping).data_ptr(), block_tables.data_ptr(),
+                block_tables.stride(0), _ptr(_i32(row_seq)), T, bs, int(pool), k_pool.shape[1], G, D, E,
+                _dt(k_cache), _stream()), "pool_block_means")
+
+
+def unturn_gate(o, positions, v_inv_freq, gate, out_dtype):
+    T, H, E = o.shape
+    assert o.stride(2) == 1 and o.dtype == out_dtype
+    if gate is not None:
+        assert gate.shape == (T, H * E) and gate.stride(1) == 1 and gate.dtype == out_dtype
+    if v_inv_freq is not None:
+        assert v_inv_freq.numel() * 2 == E
+    out = torch.empty((T, H * E), dtype=out_dtype, device=o.device)
+    _check(_utg(o.data_ptr(), o.stride(0), o.stride(1), _i32(positions).data_ptr(),
+                _ptr(_f32(v_inv_freq)) if v_inv_freq is not None else None, _ptr(gate),
+                _rows(gate) if gate is not None else 0, out.data_ptr(), T, H, E, _dt(o), _stream()),
+           "unturn_gate")
+    return out
+
+
+# ------------------------------------------------------------------ real-gated diagonal recurrence
+def short_conv(x, w, bias, conv_state, cu_q, positions, slots, row_seq):
+    T, C = x.shape
+    taps = _f32(w).shape[1]
+    assert x.stride(1) == 1 and w.shape[0] == C
+    if cu_q is not None:
+        assert row_seq is not None, "prefill-form steps pass the sequence of each row"
+    if taps > 1:
+        assert _f32(conv_state).shape[1:] == (taps - 1, C)
+    u = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    B = slots.shape[0]
+    _check(_scv(x.data_ptr(), _rows(x), w.data_ptr(), _ptr(_f32(bias)) if bias is not None else None,
+                _ptr(conv_state) if taps > 1 else None, _ptr(_i32(cu_q)), _i32(positions).data_ptr(),
+                _i32(slots).data_ptr(), _ptr(_i32(row_seq)) if cu_q is not None else None,
+                u.data_ptr(), T, B, C, taps, _dt(x), _stream()), "short_conv")
+    return u
+
+
+def scan_waves(rows: int, seqs: int, channels: int) -> int:
+    """Parts a sequence's rows are cut into by the recurrence kernel (one wave each): enough
+    workgroups x waves to fill the chip, parts of at least 32 rows."""
+    per_seq = max(1, rows // max(seqs, 1))
+    want = max(1, 4096 // max(seqs * ((channels + 63) // 64), 1))
+    return max(1, min(16, want, per_seq // 32))
+
+
+def rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp, out_dtype):
+    T, C = u.shape
+    nb = gates.shape[0]
+    assert _f32(u) is u and _f32(gates).shape == (nb, T, 2 * (C // nb)) and _f32(gate_bias).shape == (nb, 2 * (C // nb))
+    assert y.shape == (T, C) and y.stride(1) == 1 and y.dtype == out_dtype and _f32(state).shape[1] == C
+    out = torch.empty((T, C), dtype=out_dtype, device=u.device)
+    B = slots.shape[0]
+    nw = scan_waves(T, B, C) if cu_q is not None else 1
+    _check(_lru(u.data_ptr(), gates.data_ptr(), gate_bias.data_ptr(), _f32(lam).data_ptr(),
+                y.data_ptr(), _rows(y), state.data_ptr(), _ptr(_i32(cu_q)), _i32(positions).data_ptr(),
+                _i32(slots).data_ptr(), out.data_ptr(), T, B, C, nb, float(sharp), nw, _DT[out_dtype],
+                _stream()), "rglru_scan")
+    return out
+
+
+def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype):
+    T = gu.shape[0]
+    C = gu.shape[1] // 2
+    NR = dense.shape[1]
+    NE = (C - shared_ff) // ff
+    assert gu.stride(1) == 1 and gu.dtype == out_dtype and C == NE * ff + shared_ff and NR in (NE, NE + 1)
+    act = torch.empty((T, C), dtype=out_dtype, device=gu.device)
+    _check(_cgl(gu.data_ptr(), _rows(gu), _f32(dense).data_ptr(), act.data_ptr(), T, NE, NR, ff,
+                shared_ff, float(limit), float(shared_limit), _dt(gu), _stream()),
+           "capped_glu_route_scale")
+    return act

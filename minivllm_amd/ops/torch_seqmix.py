@@ -588,20 +588,22 @@ def half_rope_store(q, k, v, positions, inv_freq, rot_dims, v_inv_freq, k_cache,
         _scatter_rows(v_cache, vf, slot_mapping)
 
 
-def pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions, block_tables, row_seq):
+def pool_block_means(k_cache, v_cache, k_pool, v_pool, pool, positions, block_tables, row_seq,
+                     slot_mapping):
     """For every row of the step whose position ends a block of ``pool`` tokens (position + 1 a
     multiple of ``pool``): the means of that block's ``pool`` cached key rows and value rows
     (fp32 sums) are written to the pooled caches.  Block b of a sequence lives in row b %
     rows_per_page of page block_table[b // rows_per_page] of ``k_pool`` / ``v_pool``
     [pages, rows_per_page, G, D|E], rows_per_page * pool >= the token page size.  ``row_seq`` [T]:
     the sequence (block table row) of each row, negative for rows of no sequence; None: row t is
-    sequence t."""
+    sequence t.  Rows whose ``slot_mapping`` entry is negative (they cache nothing) are passed over."""
     bs, pr = k_cache.shape[1], k_pool.shape[1]
     pos = positions.tolist()
     seq = row_seq.tolist() if row_seq is not None else list(range(len(pos)))
+    stored = slot_mapping.tolist()
     for t, p in enumerate(pos[:len(seq)]):
         b = seq[t]
-        if b < 0 or b >= block_tables.shape[0] or (p + 1) % pool:
+        if b < 0 or stored[t] < 0 or b >= block_tables.shape[0] or (p + 1) % pool:
             continue
         table = block_tables[b]
         blk = p // pool
