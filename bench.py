@@ -359,6 +359,33 @@ def kidupel_model(size: str, vocab: int = 32768, window: int = 512):
                                     "loop": {"start": 1, "stop": 3, "times": 2}}, name=f"kidupel-{size}")
 
 
+def zegelix_model(size: str, vocab: int = 32768, experts: int = 4, top: int = 2, window: int = 512,
+                  pool: int = 64):
+    """Zegelix configuration of the same width, number of layer runs, head geometry and active
+    feed-forward parameters per token as ``hybrid_models(size)``: six layers (recurrent,
+    recurrent, attention - Griffin's two to one - twice) of which the second and third run twice,
+    i.e. eight layer runs; recurrent width 5 W / 4 in gate blocks of 128 channels, 4 taps;
+    attention over a window of ``window`` tokens with one pooled row per ``pool`` tokens behind
+    it, half of every key rotated, soft cap 30; routed capped experts plus a gated shared one
+    ((top + 1) * 3 * ff = 3 * intermediate)."""
+    from minivllm_amd.models.zegelix import ZegelixConfig
+    W, L, H, G, D, inter = HYBRID_SIZES[size]
+    ff = inter // (top + 1) // 64 * 64
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top},
+           "shared": {"ff": ff, "limit": 7.0}}
+    C = 5 * W // 4
+    kinds = [("rglru", {"width": C, "blocks": C // 128, "conv": 4}),
+             ("rglru", {"width": C, "blocks": C // 128, "conv": 4}),
+             ("attention", {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+                            "softcap": 30.0, "mask": {"size": window, "pool": pool},
+                            "rot": {"base": 10000.0, "dims": D // 2}})]
+    layers = [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": mlp} for i in range(L - 2)]
+    return ZegelixConfig.from_dict({"architecture": "Zegelix", "vocab": vocab, "width": W,
+                                    "norm": {"eps": 1e-6}, "embedding": {"scale": float(W) ** 0.5},
+                                    "logit_scale": 1.0, "layers": layers,
+                                    "loop": {"start": 1, "stop": 3, "times": 2}}, name=f"zegelix-{size}")
+
+
 def hybrid_comparison(args) -> dict:
     """Prefill and decode throughput of the hybrid families next to the dense decoder of the same
     size, one GPU, same engine path as the headline measurement (``bench_model``).
@@ -368,6 +395,8 @@ def hybrid_comparison(args) -> dict:
         return pelenex_comparison(args)
     if args.family == "kidupel":
         return kidupel_comparison(args)
+    if args.family == "zegelix":
+        return zegelix_comparison(args)
     out = {"metric": "prefill / decode tok/s, hybrid (attention + delta rule + routed experts) "
                      "next to the dense decoder of equal size",
            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -441,6 +470,35 @@ def kidupel_comparison(args) -> dict:
             if all(n in row and k in row[n] for n in ("kidupel", "pelenex", "dense")):
                 row[f"kidupel_over_pelenex_{k}"] = round(row["kidupel"][k] / row["pelenex"][k], 3)
                 row[f"kidupel_over_dense_{k}"] = round(row["kidupel"][k] / row["dense"][k], 3)
+        out["sizes"][size] = row
+    return out
+
+
+def zegelix_comparison(args) -> dict:
+    out = {"metric": "prefill / decode tok/s, Zegelix (real-gated recurrent blocks, windowed "
+                     "attention with pooled blocks, rotated values and a sink, looped layers with "
+                     "embedding re-mix, capped routed experts) next to Kidupel and the dense "
+                     "decoder of equal size",
+           "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "dtype": "bf16", "data": "synthetic random token prompts, random-init weights",
+           "config": {"seq_len": args.seq_len, "decode_batch": args.batch,
+                      "prefill_tokens_per_step": args.prefill_tokens, "kv_block_size": args.block_size},
+           "sizes": {}}
+    keep = ("prefill_tok_s", "prefill_ms_per_step", "decode_tok_s", "decode_ms_per_step",
+            "hipgraph_captured", "init_s")
+    for size in args.hybrid.split(","):
+        _, dense = hybrid_models(size)
+        row = {}
+        for name, make in (("zegelix", lambda: zegelix_model(size)), ("kidupel", lambda: kidupel_model(size)),
+                           ("dense", lambda: dense)):
+            if args.only and name != args.only:
+                continue                         # (a kernel trace of one model)
+            r = bench_model(args, make(), 0, 1)
+            row[name] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items() if k in keep}
+        for k in ("prefill_tok_s", "decode_tok_s"):
+            if all(n in row and k in row[n] for n in ("zegelix", "kidupel", "dense")):
+                row[f"zegelix_over_kidupel_{k}"] = round(row["zegelix"][k] / row["kidupel"][k], 3)
+                row[f"zegelix_over_dense_{k}"] = round(row["zegelix"][k] / row["dense"][k], 3)
         out["sizes"][size] = row
     return out
 
@@ -744,10 +802,11 @@ def main():
                          "launch floor of a real N-GPU run; NOT a scaling number)")
     ap.add_argument("--p2p", action="store_true",
                     help="with --tp-shard: all-reduces by the peer-to-peer kernels in loop-back form")
-    ap.add_argument("--family", default="natilix", choices=["natilix", "pelenex", "kidupel"],
+    ap.add_argument("--family", default="natilix", choices=["natilix", "pelenex", "kidupel", "zegelix"],
                     help="with --hybrid: which hybrid family is measured (pelenex: next to natilix "
-                         "and dense; kidupel: next to pelenex and dense)")
-    ap.add_argument("--only", default="", choices=["", "kidupel", "pelenex", "natilix", "dense"],
+                         "and dense; kidupel: next to pelenex and dense; zegelix: next to kidupel "
+                         "and dense)")
+    ap.add_argument("--only", default="", choices=["", "zegelix", "kidupel", "pelenex", "natilix", "dense"],
                     help="with --hybrid --family pelenex / kidupel: measure this one model only")
     ap.add_argument("--hybrid", default="",
                     help="instead of the headline workload: the hybrid family (Natilix) next to "

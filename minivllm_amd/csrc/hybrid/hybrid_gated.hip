@@ -73,38 +73,61 @@ __global__ void half_rope_store_kernel(T* __restrict__ q, const T* __restrict__ 
     }
 }
 
-// Grid (rows, G).  A row whose position + 1 is a multiple of `pool` completes block
-// blk = position / pool of its sequence: the fp32 sums of the block's cached rows, divided by
-// pool, go to row (table[blk / prow] * prow + blk % prow) of the pooled caches.
-template <typename T>
-__global__ void pool_block_means_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-                                        T* __restrict__ k_pool, T* __restrict__ v_pool,
-                                        const int* __restrict__ positions,
-                                        const int* __restrict__ slot_mapping,
-                                        const int* __restrict__ block_tables, int max_blocks,
-                                        const int* __restrict__ row_seq, int block_size, int pool,
-                                        int prow, int G, int D, int E) {
-    const long t = blockIdx.x;
-    const int g = blockIdx.y;
-    const int p = positions[t];
-    if (slot_mapping[t] < 0 || (p + 1) % pool) return;
-    const int b = row_seq ? row_seq[t] : (int)t;
-    if (b < 0) return;
-    const int* table = block_tables + (long)b * max_blocks;
-    const int blk = p / pool, first = blk * pool;
-    const long dst = (long)table[blk / prow] * prow + blk % prow;
+// Grid (row groups of POOL_ROWS rows, G), 256 threads.  A row whose position + 1 is a multiple of
+// `pool` completes block blk = position / pool of its sequence: the fp32 sums of the block's
+// cached rows, divided by pool, go to row (table[blk / prow] * prow + blk % prow) of the pooled
+// caches.  A thread owns VEC consecutive columns of [key | value] and every `parts`-th cached row;
+// the parts meet in LDS (parts * (D + E) floats).
+constexpr int POOL_ROWS = 8;
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+pool_block_means_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                        T* __restrict__ k_pool, T* __restrict__ v_pool,
+                        const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+                        const int* __restrict__ block_tables, int max_blocks,
+                        const int* __restrict__ row_seq, long T_, int block_size, int pool,
+                        int prow, int G, int D, int E, int parts) {
+    extern __shared__ float red[];
+    const int g = blockIdx.y, cols = D + E, cv = cols / VEC;
     const float inv = 1.f / (float)pool;
-    for (int c = threadIdx.x; c < D + E; c += blockDim.x) {
-        const bool isk = c < D;
-        const T* src = isk ? k_cache + (long)g * D + c : v_cache + (long)g * E + (c - D);
-        const long rs = isk ? (long)G * D : (long)G * E;
-        float sum = 0.f;
-        for (int j = first; j < first + pool; ++j) {
-            const long slot = (long)table[j / block_size] * block_size + j % block_size;
-            sum += ld(src + slot * rs);
+    for (int r = 0; r < POOL_ROWS; ++r) {
+        const long t = (long)blockIdx.x * POOL_ROWS + r;
+        if (t >= T_) break;
+        const int p = positions[t];
+        if (slot_mapping[t] < 0 || (p + 1) % pool) continue;            // (uniform)
+        const int b = row_seq ? row_seq[t] : (int)t;
+        if (b < 0) continue;
+        const int* table = block_tables + (long)b * max_blocks;
+        const int blk = p / pool, first = blk * pool;
+        for (int idx = threadIdx.x; idx < parts * cv; idx += blockDim.x) {
+            const int part = idx / cv, c = (idx - part * cv) * VEC;
+            const bool isk = c < D;
+            const T* src = isk ? k_cache + (long)g * D + c : v_cache + (long)g * E + (c - D);
+            const long rs = isk ? (long)G * D : (long)G * E;
+            float acc[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+            for (int j = first + part; j < first + pool; j += parts) {
+                const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                float v[VEC];
+                if constexpr (VEC == 1) v[0] = ld(src + slot * rs);
+                else load_run<T, VEC>(src + slot * rs, v);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] += v[i];
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) red[part * cols + c + i] = acc[i];
         }
-        if (isk) st(k_pool + (dst * G + g) * (long)D + c, sum * inv);
-        else st(v_pool + (dst * G + g) * (long)E + (c - D), sum * inv);
+        __syncthreads();
+        const long dst = (long)table[blk / prow] * prow + blk % prow;
+        for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+            float sum = 0.f;
+            for (int q = 0; q < parts; ++q) sum += red[q * cols + c];
+            if (c < D) st(k_pool + (dst * G + g) * (long)D + c, sum * inv);
+            else st(v_pool + (dst * G + g) * (long)E + (c - D), sum * inv);
+        }
+        __syncthreads();
     }
 }
 
@@ -151,33 +174,48 @@ __global__ void unturn_gate_kernel(const T* __restrict__ o, long o_t, long o_h,
 }
 
 // ---------------------------------------------------------------------------------------
-// u[t, c] = bias[c] + sum_k w[c, k] x(t - (taps-1-k), c); grid (rows, channel chunks).  Inputs
-// before the step's first row of the sequence come from tail [slots, taps-1, C] (the newest last);
-// positions before the sequence's start count as zeros.  Rows of no sequence give zeros.
-template <typename T>
+// u[t, c] = bias[c] + sum_k w[c, k] x(t - (taps-1-k), c); grid (rows, channel chunks); a thread owns
+// VEC consecutive channels.  Inputs before the step's first row of the sequence come from tail
+// [slots, taps-1, C] (the newest last); positions before the sequence's start count as zeros.
+// Rows of no sequence give zeros.
+template <typename T, int VEC>
 __global__ void short_conv_kernel(const T* __restrict__ x, long x_stride, const float* __restrict__ w,
                                   const float* __restrict__ bias, const float* __restrict__ tail,
                                   const int* __restrict__ cu_q, const int* __restrict__ positions,
                                   const int* __restrict__ slots, const int* __restrict__ row_seq,
                                   float* __restrict__ u, int C, int taps) {
     const long t = blockIdx.x;
-    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
     if (c >= C) return;
     const int b = cu_q ? row_seq[t] : (int)t;
     const int slot = b >= 0 ? slots[b] : -1;
-    if (slot < 0) { u[t * C + c] = 0.f; return; }
+    float acc[VEC];
+    if (slot < 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) u[t * C + c + i] = 0.f;
+        return;
+    }
     const long s0 = cu_q ? cu_q[b] : t;
     const int off = (int)(t - s0), pos = positions[t];
-    float acc = bias ? bias[c] : 0.f;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = bias ? bias[c + i] : 0.f;
     for (int k = 0; k < taps; ++k) {
         const int d = taps - 1 - k;
         if (pos - d < 0) continue;
-        float xv;
-        if (off - d >= 0) xv = ld(x + (t - d) * x_stride + c);
-        else xv = tail[((long)slot * (taps - 1) + (taps - 1 + off - d)) * C + c];
-        acc += w[(long)c * taps + k] * xv;
+        float xv[VEC];
+        if (off - d >= 0) {
+            if constexpr (VEC == 1) xv[0] = ld(x + (t - d) * x_stride + c);
+            else load_run<T, VEC>(x + (t - d) * x_stride + c, xv);
+        } else {
+            const float* tp = tail + ((long)slot * (taps - 1) + (taps - 1 + off - d)) * C + c;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) xv[i] = tp[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] += w[(long)(c + i) * taps + k] * xv[i];
     }
-    u[t * C + c] = acc;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) u[t * C + c + i] = acc[i];
 }
 
 // The kept inputs after the step: grid (channel chunks, sequences); runs after every row has read.
@@ -385,11 +423,23 @@ int hyb_pool_block_means(const void* k_cache, const void* v_cache, void* k_pool,
                          int prow, int G, int D, int E, int dt, hipStream_t s) {
     if (T_ <= 0) return 0;
     if (pool <= 0 || prow <= 0 || (long)prow * pool < block_size || !slot_mapping) return 1;
-    HYB_DISPATCH(dt, hipLaunchKernelGGL(pool_block_means_kernel<T>, dim3(T_, G), dim3(threads_for(D + E)),
-                                        0, s, (const T*)k_cache, (const T*)v_cache, (T*)k_pool,
-                                        (T*)v_pool, (const int*)positions, (const int*)slot_mapping,
-                                        (const int*)block_tables, max_blocks, (const int*)row_seq,
-                                        block_size, pool, prow, G, D, E));
+    const int esize = dt == 0 ? 2 : 4;
+    const bool vec = D % 4 == 0 && E % 4 == 0 && (size_t)k_cache % 16 == 0 && (size_t)v_cache % 16 == 0;
+    const int cv = (D + E) / (vec ? 4 : 1);
+    int parts = 256 / cv;
+    parts = parts < 1 ? 1 : (parts > pool ? pool : parts);
+    (void)esize;
+    const dim3 grid((unsigned)((T_ + POOL_ROWS - 1) / POOL_ROWS), G);
+    const size_t lds = (size_t)parts * (D + E) * sizeof(float);
+#define POOL_LAUNCH(VEC)                                                                          \
+    HYB_DISPATCH(dt, hipLaunchKernelGGL((pool_block_means_kernel<T, VEC>), grid, dim3(256), lds, s, \
+                                        (const T*)k_cache, (const T*)v_cache, (T*)k_pool,         \
+                                        (T*)v_pool, (const int*)positions,                        \
+                                        (const int*)slot_mapping, (const int*)block_tables,       \
+                                        max_blocks, (const int*)row_seq, T_, block_size, pool,    \
+                                        prow, G, D, E, parts))
+    if (vec) POOL_LAUNCH(4); else POOL_LAUNCH(1);
+#undef POOL_LAUNCH
     return HYB_LAUNCH_OK();
 }
 
@@ -411,11 +461,17 @@ int hyb_short_conv(const void* x, long x_stride, const void* w, const void* bias
                    void* u, long T_, int B, int C, int taps, int dt, hipStream_t s) {
     if (T_ <= 0 || C <= 0) return 0;
     if (taps < 1 || (cu_q && !row_seq) || (taps > 1 && !tail) || B > 65535) return 1;
+    const int esize = dt == 0 ? 2 : 4;
+    const bool vec = C % 4 == 0 && x_stride % 4 == 0 && (size_t)x % (4 * esize) == 0;
     const int th = threads_for(C), bx = (C + th - 1) / th;
-    HYB_DISPATCH(dt, hipLaunchKernelGGL(short_conv_kernel<T>, dim3(T_, bx), dim3(th), 0, s,
-                                        (const T*)x, x_stride, (const float*)w, (const float*)bias,
-                                        (const float*)tail, (const int*)cu_q, (const int*)positions,
-                                        (const int*)slots, (const int*)row_seq, (float*)u, C, taps));
+    const int thv = threads_for(C / 4), bxv = (C / 4 + thv - 1) / thv;
+#define CONV_LAUNCH(VEC, nb_, nt_)                                                                \
+    HYB_DISPATCH(dt, hipLaunchKernelGGL((short_conv_kernel<T, VEC>), dim3(T_, nb_), dim3(nt_), 0, s, \
+                                        (const T*)x, x_stride, (const float*)w, (const float*)bias, \
+                                        (const float*)tail, (const int*)cu_q, (const int*)positions, \
+                                        (const int*)slots, (const int*)row_seq, (float*)u, C, taps))
+    if (vec) CONV_LAUNCH(4, bxv, thv); else CONV_LAUNCH(1, bx, th);
+#undef CONV_LAUNCH
     if (hipGetLastError() != hipSuccess) return 2;
     if (taps > 1 && B > 0)
         HYB_DISPATCH(dt, hipLaunchKernelGGL(short_conv_tail_kernel<T>, dim3(bx, B), dim3(th), 0, s,

@@ -669,8 +669,9 @@ def rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp
     g = torch.sigmoid(gates.float() + gate_bias.float()[:, None, :])          # [nb, T, 2c]
     r = g[:, :, :c].permute(1, 0, 2).reshape(T, C)
     i = g[:, :, c:].permute(1, 0, 2).reshape(T, C)
-    d = torch.exp(-sharp * r * F.softplus(lam.float()))
-    add = torch.sqrt(1.0 - d * d) * i * u
+    la = -sharp * r * F.softplus(lam.float())                 # log of the decay
+    d = torch.exp(la)
+    add = torch.sqrt(-torch.expm1(2.0 * la)) * i * u          # sqrt(1 - d^2), exact next to d = 1
     out = torch.zeros(T, C, dtype=torch.float32)
     for s, e, slot, past in _seq_rows(cu_q, positions, slots):
         S = state[slot].clone() if past else torch.zeros(C)
