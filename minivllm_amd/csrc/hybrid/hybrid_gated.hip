@@ -174,48 +174,78 @@ __global__ void unturn_gate_kernel(const T* __restrict__ o, long o_t, long o_h,
 }
 
 // ---------------------------------------------------------------------------------------
-// u[t, c] = bias[c] + sum_k w[c, k] x(t - (taps-1-k), c); grid (rows, channel chunks); a thread owns
-// VEC consecutive channels.  Inputs before the step's first row of the sequence come from tail
-// [slots, taps-1, C] (the newest last); positions before the sequence's start count as zeros.
-// Rows of no sequence give zeros.
+// u[t, c] = bias[c] + sum_k w[c, k] x(t - (taps-1-k), c); grid (groups of CONV_ROWS rows, channel
+// chunks); a thread owns VEC consecutive channels, keeps their taps (up to CONV_TAPS; longer filters
+// read them from memory) in registers and walks the group's rows.  Inputs before the step's first
+// row of the sequence come from tail [slots, taps-1, C] (the newest last); positions before the
+// sequence's start count as zeros.  Rows of no sequence give zeros.
+constexpr int CONV_ROWS = 8, CONV_TAPS = 8;
+
 template <typename T, int VEC>
 __global__ void short_conv_kernel(const T* __restrict__ x, long x_stride, const float* __restrict__ w,
                                   const float* __restrict__ bias, const float* __restrict__ tail,
                                   const int* __restrict__ cu_q, const int* __restrict__ positions,
                                   const int* __restrict__ slots, const int* __restrict__ row_seq,
-                                  float* __restrict__ u, int C, int taps) {
-    const long t = blockIdx.x;
+                                  float* __restrict__ u, long T_, int C, int taps) {
     const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
     if (c >= C) return;
-    const int b = cu_q ? row_seq[t] : (int)t;
-    const int slot = b >= 0 ? slots[b] : -1;
-    float acc[VEC];
-    if (slot < 0) {
+    float wr[VEC][CONV_TAPS], b0[VEC];
+    const bool inreg = taps <= CONV_TAPS;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) u[t * C + c + i] = 0.f;
-        return;
+    for (int i = 0; i < VEC; ++i) {
+        b0[i] = bias ? bias[c + i] : 0.f;
+#pragma unroll
+        for (int k = 0; k < CONV_TAPS; ++k) wr[i][k] = (inreg && k < taps) ? w[(long)(c + i) * taps + k] : 0.f;
     }
-    const long s0 = cu_q ? cu_q[b] : t;
-    const int off = (int)(t - s0), pos = positions[t];
+    for (int r = 0; r < CONV_ROWS; ++r) {
+        const long t = (long)blockIdx.x * CONV_ROWS + r;
+        if (t >= T_) return;
+        const int b = cu_q ? row_seq[t] : (int)t;
+        const int slot = b >= 0 ? slots[b] : -1;
+        float acc[VEC];
+        if (slot < 0) {
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = bias ? bias[c + i] : 0.f;
-    for (int k = 0; k < taps; ++k) {
-        const int d = taps - 1 - k;
-        if (pos - d < 0) continue;
-        float xv[VEC];
-        if (off - d >= 0) {
-            if constexpr (VEC == 1) xv[0] = ld(x + (t - d) * x_stride + c);
-            else load_run<T, VEC>(x + (t - d) * x_stride + c, xv);
+            for (int i = 0; i < VEC; ++i) u[t * C + c + i] = 0.f;
+            continue;
+        }
+        const long s0 = cu_q ? cu_q[b] : t;
+        const int off = (int)(t - s0), pos = positions[t];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = b0[i];
+        auto input = [&](int d, float* xv) {
+            if (off - d >= 0) {
+                if constexpr (VEC == 1) xv[0] = ld(x + (t - d) * x_stride + c);
+                else load_run<T, VEC>(x + (t - d) * x_stride + c, xv);
+            } else {
+                const float* tp = tail + ((long)slot * (taps - 1) + (taps - 1 + off - d)) * C + c;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) xv[i] = tp[i];
+            }
+        };
+        if (inreg) {
+#pragma unroll
+            for (int k = 0; k < CONV_TAPS; ++k) {
+                const int d = taps - 1 - k;
+                if (k < taps && pos - d >= 0) {
+                    float xv[VEC];
+                    input(d, xv);
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) acc[i] += wr[i][k] * xv[i];
+                }
+            }
         } else {
-            const float* tp = tail + ((long)slot * (taps - 1) + (taps - 1 + off - d)) * C + c;
+            for (int k = 0; k < taps; ++k) {
+                const int d = taps - 1 - k;
+                if (pos - d < 0) continue;
+                float xv[VEC];
+                input(d, xv);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) xv[i] = tp[i];
+                for (int i = 0; i < VEC; ++i) acc[i] += w[(long)(c + i) * taps + k] * xv[i];
+            }
         }
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) acc[i] += w[(long)(c + i) * taps + k] * xv[i];
+        for (int i = 0; i < VEC; ++i) u[t * C + c + i] = acc[i];
     }
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) u[t * C + c + i] = acc[i];
 }
 
 // The kept inputs after the step: grid (channel chunks, sequences); runs after every row has read.
@@ -466,10 +496,12 @@ int hyb_short_conv(const void* x, long x_stride, const void* w, const void* bias
     const int th = threads_for(C), bx = (C + th - 1) / th;
     const int thv = threads_for(C / 4), bxv = (C / 4 + thv - 1) / thv;
 #define CONV_LAUNCH(VEC, nb_, nt_)                                                                \
-    HYB_DISPATCH(dt, hipLaunchKernelGGL((short_conv_kernel<T, VEC>), dim3(T_, nb_), dim3(nt_), 0, s, \
+    HYB_DISPATCH(dt, hipLaunchKernelGGL((short_conv_kernel<T, VEC>),                              \
+                                        dim3((unsigned)((T_ + CONV_ROWS - 1) / CONV_ROWS), nb_),  \
+                                        dim3(nt_), 0, s,                                          \
                                         (const T*)x, x_stride, (const float*)w, (const float*)bias, \
                                         (const float*)tail, (const int*)cu_q, (const int*)positions, \
-                                        (const int*)slots, (const int*)row_seq, (float*)u, C, taps))
+                                        (const int*)slots, (const int*)row_seq, (float*)u, T_, C, taps))
     if (vec) CONV_LAUNCH(4, bxv, thv); else CONV_LAUNCH(1, bx, th);
 #undef CONV_LAUNCH
     if (hipGetLastError() != hipSuccess) return 2;

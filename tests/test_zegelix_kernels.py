@@ -172,7 +172,7 @@ def test_attention_with_pooled_blocks(dt, H, G, D, E, bs, window, pool, cap):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("C,nb,taps", [(72, 6, 4), (192, 1, 1), (130, 2, 3)])
+@pytest.mark.parametrize("C,nb,taps", [(72, 6, 4), (192, 1, 1), (130, 2, 3), (96, 3, 9)])
 def test_conv_and_recurrence_over_steps(dt, C, nb, taps):
     torch.manual_seed(4)
     c = C // nb
