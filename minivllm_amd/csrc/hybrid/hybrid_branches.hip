@@ -151,23 +151,6 @@ __global__ void latent_rope_store_kernel(const T* __restrict__ q_abs, const T* _
     }
 }
 
-// eight consecutive elements narrowed from fp32 and stored as one run (16 bytes of bfloat16, two
-// 16-byte stores of float); the address must be aligned to the run
-template <typename T> __device__ __forceinline__ void store_run8(T* p, const float* v);
-template <> __device__ __forceinline__ void store_run8<float>(float* p, const float* v) {
-    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
-}
-template <> __device__ __forceinline__ void store_run8<bf16_t>(bf16_t* p, const float* v) {
-    uint32_t w[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const __bf16 lo = (__bf16)v[2 * i], hi = (__bf16)v[2 * i + 1];
-        w[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
-    }
-    *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
-}
-
 __device__ __forceinline__ float xielu_(float z, float above, float below) {
     return z > 0.f ? above * z * z + 0.5f * z : below * (expm1f(z) - z) + 0.5f * z;
 }

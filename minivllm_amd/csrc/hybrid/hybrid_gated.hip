@@ -108,6 +108,7 @@ pool_block_means_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_c
             float acc[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+#pragma unroll 8
             for (int j = first + part; j < first + pool; j += parts) {
                 const long slot = (long)table[j / block_size] * block_size + j % block_size;
                 float v[VEC];
@@ -132,12 +133,14 @@ pool_block_means_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_c
 }
 
 // out[t, h*E + m] = turned-back o[t, h, :] * sigmoid(gate[t, h*E + m]); o with strides (o_t, o_h, 1).
+// vec: E/2 is a multiple of eight and every row 16-byte addressable - a thread then moves runs of
+// eight columns of both halves of a head.
 template <typename T>
 __global__ void unturn_gate_kernel(const T* __restrict__ o, long o_t, long o_h,
                                    const int* __restrict__ positions,
                                    const float* __restrict__ v_inv_freq,
                                    const T* __restrict__ gate, long gate_stride,
-                                   T* __restrict__ out, int H, int E) {
+                                   T* __restrict__ out, int H, int E, int vec) {
     extern __shared__ float sm[];
     const long t = blockIdx.x;
     const int half = E / 2;
@@ -152,7 +155,27 @@ __global__ void unturn_gate_kernel(const T* __restrict__ o, long o_t, long o_h,
     }
     const T* gr = gate ? gate + t * gate_stride : nullptr;
     T* orow = out + t * (long)(H * E);
-    if (v_inv_freq) {
+    if (v_inv_freq && vec) {
+        const int runs = half / 8;
+        for (int i = threadIdx.x; i < H * runs; i += blockDim.x) {
+            const int h = i / runs, m = (i - h * runs) * 8;
+            const T* a = o + t * o_t + (long)h * o_h + m;
+            float u[8], w[8], gu[8], gw[8], x[8], y[8];
+            load_run<T, 8>(a, u);
+            load_run<T, 8>(a + half, w);
+            const int col = h * E + m;
+            if (gr) { load_run<T, 8>(gr + col, gu); load_run<T, 8>(gr + col + half, gw); }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float c = sm[m + j], s = sm[half + m + j];
+                x[j] = u[j] * c + w[j] * s;
+                y[j] = w[j] * c - u[j] * s;
+                if (gr) { x[j] *= sigmoidf_(gu[j]); y[j] *= sigmoidf_(gw[j]); }
+            }
+            store_run8<T>(orow + col, x);
+            store_run8<T>(orow + col + half, y);
+        }
+    } else if (v_inv_freq) {
         for (int i = threadIdx.x; i < H * half; i += blockDim.x) {
             const int h = i / half, m = i - h * half;
             const T* a = o + t * o_t + (long)h * o_h + m;
@@ -176,7 +199,8 @@ __global__ void unturn_gate_kernel(const T* __restrict__ o, long o_t, long o_h,
 // ---------------------------------------------------------------------------------------
 // u[t, c] = bias[c] + sum_k w[c, k] x(t - (taps-1-k), c); grid (groups of CONV_ROWS rows, channel
 // chunks); a thread owns VEC consecutive channels, keeps their taps (up to CONV_TAPS; longer filters
-// read them from memory) in registers and walks the group's rows.  Inputs before the step's first
+// read them from memory) in registers and walks the group's `rows_per` rows (CONV_ROWS for prompt
+// portions, one for a handful of single tokens).  Inputs before the step's first
 // row of the sequence come from tail [slots, taps-1, C] (the newest last); positions before the
 // sequence's start count as zeros.  Rows of no sequence give zeros.
 constexpr int CONV_ROWS = 8, CONV_TAPS = 8;
@@ -186,7 +210,7 @@ __global__ void short_conv_kernel(const T* __restrict__ x, long x_stride, const 
                                   const float* __restrict__ bias, const float* __restrict__ tail,
                                   const int* __restrict__ cu_q, const int* __restrict__ positions,
                                   const int* __restrict__ slots, const int* __restrict__ row_seq,
-                                  float* __restrict__ u, long T_, int C, int taps) {
+                                  float* __restrict__ u, long T_, int C, int taps, int rows_per) {
     const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
     if (c >= C) return;
     float wr[VEC][CONV_TAPS], b0[VEC];
@@ -197,8 +221,8 @@ __global__ void short_conv_kernel(const T* __restrict__ x, long x_stride, const 
 #pragma unroll
         for (int k = 0; k < CONV_TAPS; ++k) wr[i][k] = (inreg && k < taps) ? w[(long)(c + i) * taps + k] : 0.f;
     }
-    for (int r = 0; r < CONV_ROWS; ++r) {
-        const long t = (long)blockIdx.x * CONV_ROWS + r;
+    for (int r = 0; r < rows_per; ++r) {
+        const long t = (long)blockIdx.x * rows_per + r;
         if (t >= T_) return;
         const int b = cu_q ? row_seq[t] : (int)t;
         const int slot = b >= 0 ? slots[b] : -1;
@@ -272,8 +296,20 @@ __global__ void short_conv_tail_kernel(const T* __restrict__ x, long x_stride, f
     }
 }
 
+// sigmoid on the hardware exponential and reciprocal (both within a few ulp): the scan evaluates
+// three per element and pass
+__device__ __forceinline__ float fast_sigmoid(float z) { return __fdividef(1.f, 1.f + __expf(-z)); }
+
+// 0.5 z (1 + tanh(a)) = z sigmoid(2 a), a = sqrt(2/pi) (z + 0.044715 z^3)
 __device__ __forceinline__ float gelu_tanh_(float z) {
-    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z * fast_sigmoid(1.5957691216057308f * (z + 0.044715f * z * z * z));
+}
+
+// 1 - exp(t) for t <= 0 without cancellation: the series next to zero, 1 - exp(t) elsewhere
+__device__ __forceinline__ float one_minus_exp(float t, float e) {
+    const float series = -t * (1.f + t * (0.5f + t * (1.f / 6.f + t * (1.f / 24.f + t * (1.f / 120.f +
+                               t * (1.f / 720.f + t * (1.f / 5040.f)))))));
+    return t > -0.25f ? series : 1.f - e;
 }
 
 // Workgroup = 64 channels x nw waves of one sequence; wave w walks the w-th part of the
@@ -287,11 +323,11 @@ __device__ __forceinline__ GateStep rglru_step(const float* __restrict__ gates, 
                                                long t, long T_, int C, int c2, long gcol, int ch,
                                                float br, float bi, float nsp) {
     const float* gp = gates + t * c2 + gcol;
-    const float r = sigmoidf_(gp[0] + br), i = sigmoidf_(gp[c2 / 2] + bi);
+    const float r = fast_sigmoid(gp[0] + br), i = fast_sigmoid(gp[c2 / 2] + bi);
     const float la = nsp * r;                                   // log of the decay
     GateStep s;
-    s.d = expf(la);
-    s.add = sqrtf(-expm1f(2.f * la)) * i * u[t * C + ch];      // sqrt(1 - d^2)
+    s.d = __expf(la);
+    s.add = sqrtf(one_minus_exp(2.f * la, s.d * s.d)) * i * u[t * C + ch];      // sqrt(1 - d^2)
     return s;
 }
 
@@ -478,10 +514,13 @@ int hyb_unturn_gate(const void* o, long o_t, long o_h, const void* positions, co
                     hipStream_t s) {
     if (T_ <= 0) return 0;
     if (v_inv_freq && E % 2) return 1;
-    HYB_DISPATCH(dt, hipLaunchKernelGGL(unturn_gate_kernel<T>, dim3(T_), dim3(threads_for(H * E / 2)),
+    const int vec = v_inv_freq && E % 16 == 0 && o_t % 8 == 0 && o_h % 8 == 0 && gate_stride % 8 == 0 &&
+                    ((size_t)o | (size_t)gate | (size_t)out) % 16 == 0;
+    HYB_DISPATCH(dt, hipLaunchKernelGGL(unturn_gate_kernel<T>, dim3(T_),
+                                        dim3(threads_for(vec ? H * E / 16 : H * E / 2)),
                                         (E + 1) * sizeof(float), s, (const T*)o, o_t, o_h,
                                         (const int*)positions, (const float*)v_inv_freq,
-                                        (const T*)gate, gate_stride, (T*)out, H, E));
+                                        (const T*)gate, gate_stride, (T*)out, H, E, vec));
     return HYB_LAUNCH_OK();
 }
 
@@ -495,13 +534,15 @@ int hyb_short_conv(const void* x, long x_stride, const void* w, const void* bias
     const bool vec = C % 4 == 0 && x_stride % 4 == 0 && (size_t)x % (4 * esize) == 0;
     const int th = threads_for(C), bx = (C + th - 1) / th;
     const int thv = threads_for(C / 4), bxv = (C / 4 + thv - 1) / thv;
+    const int rows_per = T_ >= 2048 ? CONV_ROWS : 1;
 #define CONV_LAUNCH(VEC, nb_, nt_)                                                                \
     HYB_DISPATCH(dt, hipLaunchKernelGGL((short_conv_kernel<T, VEC>),                              \
-                                        dim3((unsigned)((T_ + CONV_ROWS - 1) / CONV_ROWS), nb_),  \
+                                        dim3((unsigned)((T_ + rows_per - 1) / rows_per), nb_),    \
                                         dim3(nt_), 0, s,                                          \
                                         (const T*)x, x_stride, (const float*)w, (const float*)bias, \
                                         (const float*)tail, (const int*)cu_q, (const int*)positions, \
-                                        (const int*)slots, (const int*)row_seq, (float*)u, T_, C, taps))
+                                        (const int*)slots, (const int*)row_seq, (float*)u, T_, C, taps, \
+                                        rows_per))
     if (vec) CONV_LAUNCH(4, bxv, thv); else CONV_LAUNCH(1, bx, th);
 #undef CONV_LAUNCH
     if (hipGetLastError() != hipSuccess) return 2;

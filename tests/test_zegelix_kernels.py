@@ -39,7 +39,7 @@ def paged(n, rows, extra_rows, G, d, dt, device):
 def test_rotation_store_and_turn_back(dt, H, G, D, E, dims):
     torch.manual_seed(0)
     T, bs, nb = 21, 8, 6
-    proj = torch.randn(T, H * D + G * D + G * E + H * E + 3).to(dt)
+    proj = torch.randn(T, H * D + G * D + G * E + H * E + 8).to(dt)
     pos = torch.randint(0, 3000, (T,), dtype=torch.int32)
     pos[0] = 0
     slots = torch.randperm(nb * bs)[:T].to(torch.int32)
@@ -48,7 +48,7 @@ def test_rotation_store_and_turn_back(dt, H, G, D, E, dims):
     out = {}
     for name, mod, to in (("cpu", ref, lambda t: t), ("gpu", hk, lambda t: None if t is None else t.cuda())):
         p = to(proj.clone())
-        q, k, v, g, _ = p.split([H * D, G * D, G * E, H * E, 3], -1)
+        q, k, v, g, _ = p.split([H * D, G * D, G * E, H * E, 8], -1)
         kc, vc = to(torch.zeros(nb, bs, G, D, dtype=dt)), to(torch.zeros(nb, bs, G, E, dtype=dt))
         mod.half_rope_store(q.view(T, H, D), k.view(T, G, D), v.view(T, G, E), to(pos), to(f), dims,
                             to(vf), kc, vc, to(slots))
