@@ -97,7 +97,7 @@ ALONE = {
     "attention-no-cap-pool-of-one": ([(fx.attention(heads=3, kv_heads=3, dim=16, vdim=4, size=6, pool=1,
                                                     softcap=0.0, rot_dims=2), None)], None),
     "attention-serving-sizes": ([(fx.attention(heads=4, kv_heads=2, dim=64, vdim=64, size=10, pool=3,
-                                               rot_dims=32, scale=0.125), None)], None),
+                                               rot_dims=32, scale=0.11), None)], None),
     "experts": ([(fx.rglru(width=8, blocks=1, conv=1), fx.moe())], None),
     "experts-no-shared": ([(fx.rglru(width=8, blocks=1, conv=1), fx.moe(experts=6, top=3, ff=8, shared_ff=0))], None),
     "one-layer-three-times": ([(fx.rglru(), fx.moe(ff=8))], (0, 1, 3)),

@@ -139,6 +139,8 @@ def _to_gpu(c, dt, G, D, E, bs):
     (4, 2, 128, 64, 64, 33, 5, 0.0),       # pooled rows that straddle pages, no cap
     (4, 4, 24, 20, 8, 7, 3, 2.0),          # sizes without a tile or split instance: row kernel
     (8, 2, 64, 128, 32, 50, 0, 5.0),       # no pooled blocks: window, cap and temperatures alone
+    (12, 2, 64, 64, 16, 21, 4, 0.0),       # six query heads per KV head: two groups of heads per workgroup
+    (8, 1, 32, 32, 16, 9, 2, 4.0),         # padded tile instance, row kernel for single tokens
 ])
 def test_attention_with_pooled_blocks(dt, H, G, D, E, bs, window, pool, cap):
     lens, qlens = [300, 97, 41, 130], [300, 30, 2, 129]
