@@ -176,8 +176,8 @@ class SinkAttention(nn.Module):
     on the scaled score (``temps`` [H] fp32); ``softcap`` > 0 - score <- softcap tanh(score /
     softcap) after scale and temperature; ``pool`` > 0 (needs a window) - besides the window's
     tokens a query at position i sees ONE key and value for every block of ``pool`` tokens that
-    has passed out of its window as a whole (b pool + pool - 1 <= i - window): the means of the block's
-    cached keys and values, kept in ``k_pool`` / ``v_pool`` [pages, rows, G, D|E] that the engine
+    has passed out of its window as a whole (b pool + pool - 1 <= i - window): the means of the
+    block's cached keys and values, kept in ``k_pool`` / ``v_pool`` [pages, rows, G, D|E] that the engine
     allocates next to the token caches (``block_cache_spec``) and ``update_pools`` fills once the
     step's tokens are cached; block rows and token rows are weighed in the same softmax."""
 

@@ -269,7 +269,8 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
                            k_pool=None, v_pool=None):
     """``temps`` [H] fp32: a score multiplier per head; ``softcap`` > 0: score <- softcap
     tanh(score / softcap); ``pool`` > 0 with ``k_pool`` / ``v_pool``: one pooled key / value per
-    block of ``pool`` tokens that has passed out of the window as a whole (``ops.pool_block_means``).
+    block of ``pool`` tokens that has passed out of the window as a whole
+    (``ops.pool_block_means``).
     ``positions`` [T], ``max_q`` (longest portion, a host integer), ``row_seq`` and ``first_seq``
     (how many sequences of the step precede ``cu_q[0]``'s, i.e. what was sliced off): what the
     GPU kernels take besides (``hip_hybrid.sink_attention_prefill``); the CPU form derives

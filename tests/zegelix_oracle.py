@@ -15,8 +15,9 @@ The design in this file's notation (W = width, every norm is x / sqrt(mean(x^2) 
   and k turned in half-split pairs by p f_m, f_m = base^(-2m/dims); values turned over ALL their
   entries by j f'_m, f'_m = base^(-2m/E), before they are cached, each head's weighted sum turned
   back by the query's position; score = cap tanh(scale temp_h (q . k) / cap); query i sees tokens
-  j with 0 <= i - j < size and, for every block of P tokens that has passed out of that window as a whole
-  (bP + P - 1 <= i - size), ONE key and value, the means of the block's cached keys and values;
+  j with 0 <= i - j < size and, for every block of P tokens that has passed out of that window as
+  a whole (bP + P - 1 <= i - size), ONE key and value, the means of the block's cached keys and
+  values;
   one softmax over tokens and blocks whose denominator also holds exp(sink_h); the heads' outputs
   times sigmoid(G_w h) element by element, then the output projection;
 * ff: router logits z = R h + r; the `top` largest are chosen, weights = softmax over those;
@@ -56,7 +57,8 @@ def turn_halves(x, position, base, dims, sign=1.0):
 
 
 def causal_filter(x, taps_w, bias):
-    """x [T, C]; taps_w [C, taps], the last column meets the current token and nothing precedes a sequence."""
+    """x [T, C]; taps_w [C, taps], the last column meets the current token and nothing precedes
+    a sequence."""
     T, C = x.shape
     taps = taps_w.shape[1]
     out = torch.zeros(T, C, dtype=F64)
