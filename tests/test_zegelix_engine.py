@@ -464,3 +464,17 @@ def test_checkpoint_errors_name_the_tensor(tmp_path):
     del bad["l0.mlp.shared.sg"]
     with pytest.raises(KeyError, match="l0.mlp.shared.sg"):
         make_engine(tmp_path / "u", c, bad, "cpu", "float32")
+
+
+def test_benchmark_configuration_parses_and_validates():
+    import types
+    sys.path.insert(0, ROOT)
+    import bench
+    for size in ("w1024", "w2048"):
+        mc = bench.zegelix_model(size)
+        mc.validate_engine(types.SimpleNamespace(tp_degree=1))
+        runs = mc.run_order()
+        assert len(runs) == 8 and sum(first for _, _, first in runs) == 2
+        assert [mc.layers[i].type for i, _, _ in runs].count("attention") == 3
+    with pytest.raises(ValueError, match="one rank"):
+        mc.validate_engine(types.SimpleNamespace(tp_degree=2))
