@@ -245,7 +245,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 // 16-bit K tile and q rows - the operands ARE bfloat16 values, so the products are exact and the
 // fp32 accumulation only differs in order from the fp32 instruction; the score scale is applied
 // to the fp32 result.  Weights and weighted sums stay on the fp32 instruction.
-template <typename T, int DP, int EP, bool QK16>
+// EXT: the instance that knows head temperatures, the soft cap and pooled rows; without it the
+// kernel is compiled free of them (their state costs registers the plain form has no room for).
+template <typename T, int DP, int EP, bool QK16, bool EXT>
 __global__ void __launch_bounds__(256)
 sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                             const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -271,7 +273,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
     const bool qok = qi < qlen;
     const int qpos = start + qi;
 
-    const float hscale = rule.head_scale(scale, h);
+    const float hscale = EXT ? rule.head_scale(scale, h) : scale;
     float qreg[QK16 ? 1 : DP / 2];
     bf16x8 qv[QK16 ? DP / 16 : 1];
     {
@@ -316,10 +318,10 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
     const int wave_lo = rule.window > 0 ? max(0, start + tile * 128 + wave * 32 - rule.window + 1) : 0;
 
     // pooled rows first (those the workgroup's last query takes in), then the tokens
-    const int wg_nb = rule.pooled_for(wg_ctx), ptiles = (wg_nb + 31) / 32;
-    const int wave_nb = rule.pooled_for(wave_last + 1), q_nb = rule.pooled_for(qpos + 1);
+    const int wg_nb = EXT ? rule.pooled_for(wg_ctx) : 0, ptiles = EXT ? (wg_nb + 31) / 32 : 0;
+    const int wave_nb = EXT ? rule.pooled_for(wave_last + 1) : 0, q_nb = EXT ? rule.pooled_for(qpos + 1) : 0;
     for (int it = 0; it < ptiles + (wg_ctx + 31) / 32; ++it) {
-        const bool pooled = it < ptiles;                              // (uniform)
+        const bool pooled = EXT && it < ptiles;                       // (uniform)
         const int k0 = (pooled ? it : it - ptiles) * 32;
         const int k_lim = pooled ? wg_nb : wg_ctx;
         if (!pooled && k0 >= rule.keep_first && k0 + 32 <= wg_lo) continue;   // (uniform) nobody sees this tile
@@ -412,7 +414,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                 const int key = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
                 const bool seen = qok && (pooled ? key < q_nb : (key <= qpos &&
                                   (rule.window <= 0 || qpos - key < rule.window || key < rule.keep_first)));
-                const float v = seen ? rule.capped(sacc[r]) - (pooled ? 0.f : slope * (float)(qpos - key)) : -INFINITY;
+                const float v = seen ? (EXT ? rule.capped(sacc[r]) : sacc[r]) - (pooled ? 0.f : slope * (float)(qpos - key)) : -INFINITY;
                 sacc[r] = v;
                 mt = fmaxf(mt, v);
             }
@@ -466,12 +468,15 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
     const int vec_k = (D % 4 == 0) && ((size_t)k_cache % 16 == 0);
     const int vec_v = (E % 4 == 0) && (rule.v_stride % 4 == 0) && ((size_t)v_cache % 16 == 0);
     const dim3 grid(nseq, (max_q + 127) / 128, H);
-#define TILES_LAUNCH(QK16, lds)                                                                   \
-    hipLaunchKernelGGL((sink_attention_tiles_kernel<T, DP, EP, QK16>), grid, dim3(256), lds, s,   \
+#define TILES_LAUNCH_X(QK16, EXT, lds)                                                            \
+    hipLaunchKernelGGL((sink_attention_tiles_kernel<T, DP, EP, QK16, EXT>), grid, dim3(256), lds, s, \
                        (const T*)q, q_row, q_head, (const T*)k_cache, (const T*)v_cache,          \
                        (const int*)block_tables, max_blocks, block_size, (const int*)cu_q,        \
                        (const int*)positions, (const float*)sink, (const T*)gate, gate_row,       \
                        (T*)out, scale, H, G, D, E, seq0, vec_k, vec_v, rule)
+#define TILES_LAUNCH(QK16, lds)                                                                   \
+    do { if (ext) TILES_LAUNCH_X(QK16, true, lds); else TILES_LAUNCH_X(QK16, false, lds); } while (0)
+    const bool ext = rule.temps || rule.softcap > 0.f || rule.pool > 0;
     if constexpr (sizeof(T) == 2) {
         // 16-bit caches: score products on the bf16 instruction when rows are 16-byte addressable
         if (D % 16 == 0 && (size_t)k_cache % 16 == 0 && (size_t)q % 16 == 0 && q_row % 8 == 0 &&
@@ -482,6 +487,7 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
     }
     TILES_LAUNCH(false, (32 * (DP + 1) + 32 * EP) * sizeof(float));
 #undef TILES_LAUNCH
+#undef TILES_LAUNCH_X
     return HYB_LAUNCH_OK();
 }
 
@@ -493,7 +499,7 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
 // the groups' partials meet in LDS, the workgroups' (one per context split) in a workspace that
 // `sink_attention_merge_kernel` folds together with the sink term and the gate.
 // EPL / VPL: elements of a K / V row per lane (D = 16 EPL, E = 16 VPL).
-template <typename T, int EPL, int VPL>
+template <typename T, int EPL, int VPL, bool EXT>
 __global__ void __launch_bounds__(256)
 sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
                             const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -519,7 +525,7 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
     for (int r = 0; r < RC; ++r) {
         if (r < nr) {
             load_run<T, EPL>(q + b * q_row + (long)(h0 + r) * q_head + lane16 * EPL, qf[r]);
-            const float hs = rule.head_scale(scale, h0 + r);
+            const float hs = EXT ? rule.head_scale(scale, h0 + r) : scale;
 #pragma unroll
             for (int i = 0; i < EPL; ++i) qf[r][i] *= hs;
             m[r] = sink ? sink[h0 + r] : NO_SINK_MAX;
@@ -539,8 +545,10 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
         const bool two = vj + 16 < k_end;
         const int j = vis.key(vj), j2 = two ? vis.key(vj + 16) : j;
         const float dist[2] = {(float)(ctx - 1 - j), (float)(ctx - 1 - j2)};
-        const long slot = vis.row(vj, table, block_size, rule);
-        const long slot2 = two ? vis.row(vj + 16, table, block_size, rule) : slot;
+        const long slot = EXT ? vis.row(vj, table, block_size, rule)
+                              : (long)table[j / block_size] * block_size + j % block_size;
+        const long slot2 = !two ? slot : EXT ? vis.row(vj + 16, table, block_size, rule)
+                                             : (long)table[j2 / block_size] * block_size + j2 % block_size;
         float kf[2][EPL], vf[2][VPL];
         load_run<T, EPL>(k_cache + (slot * G + g) * (long)D + lane16 * EPL, kf[0]);
         load_run<T, EPL>(k_cache + (slot2 * G + g) * (long)D + lane16 * EPL, kf[1]);
@@ -559,7 +567,7 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
                 d += __shfl_xor(d, 2, kWave);
                 d += __shfl_xor(d, 4, kWave);
                 d += __shfl_xor(d, 8, kWave);
-                d = rule.capped(d) - slope[r] * dist[x];
+                d = (EXT ? rule.capped(d) : d) - slope[r] * dist[x];
                 if (d > m[r]) {                    // the running maximum moves: rescale (rare)
                     const float a = expf(m[r] - d);
                     l[r] *= a;
@@ -633,11 +641,14 @@ static int launch_split(const void* q, long q_row, long q_head, const void* k_ca
     constexpr int E = 16 * VPL;
     const int R = H / G, chunks = (R + RC - 1) / RC;
     const size_t lds = 16 * RC * (E + 2) * sizeof(float);
-    hipLaunchKernelGGL((sink_attention_split_kernel<T, EPL, VPL>), dim3(B, G * chunks, splits),
-                       dim3(256), lds, s, (const T*)q, q_row, q_head, (const T*)k_cache,
-                       (const T*)v_cache, (const int*)block_tables, max_blocks, block_size,
-                       (const int*)context_lens, (const float*)sink, (float*)ws, scale, H, G, splits,
-                       rule);
+#define SPLIT_LAUNCH(EXT)                                                                         \
+    hipLaunchKernelGGL((sink_attention_split_kernel<T, EPL, VPL, EXT>), dim3(B, G * chunks, splits), \
+                       dim3(256), lds, s, (const T*)q, q_row, q_head, (const T*)k_cache,          \
+                       (const T*)v_cache, (const int*)block_tables, max_blocks, block_size,       \
+                       (const int*)context_lens, (const float*)sink, (float*)ws, scale, H, G, splits, \
+                       rule)
+    if (rule.temps || rule.softcap > 0.f || rule.pool > 0) SPLIT_LAUNCH(true); else SPLIT_LAUNCH(false);
+#undef SPLIT_LAUNCH
     if (hipGetLastError() != hipSuccess) return 2;
     hipLaunchKernelGGL(sink_attention_merge_kernel<T>, dim3(B * H), dim3(E >= 128 ? 128 : 64), 0, s,
                        (const float*)ws, (const float*)sink, (const T*)gate, gate_row,
