@@ -7,7 +7,7 @@
 //   short_conv (+ tail)     causal per-channel filter over a step's rows and a sequence's kept inputs
 //   rglru_scan              S <- d S + sqrt(1 - d^2) i u per channel, output S * gelu_tanh(y)
 //   chosen_route            router logits + bias, top logits, softmax over the chosen, gate rows
-//   capped_glu_route_scale  w * min(g, L) sigmoid(1.702 min(g, L)) (clamp(u, -L, L) + 1)
+//   capped_glu_route_scale  w * min(g, L) sigmoid(slope min(g, L)) (clamp(u, -L, L) + 1)
 // Angles, gates, decays, state, router and every transcendental in fp32.
 #include "hybrid_common.h"
 
@@ -437,7 +437,7 @@ template <typename T, int VEC>
 __global__ void capped_glu_route_scale_kernel(const T* __restrict__ gu, long gu_stride,
                                               const float* __restrict__ dense, T* __restrict__ act,
                                               int NE, int NR, int ff, int C, float limit,
-                                              float shared_limit) {
+                                              float shared_limit, float slope) {
     const long t = blockIdx.y;
     const T* g = gu + t * gu_stride;
     const T* u = g + C;
@@ -453,7 +453,7 @@ __global__ void capped_glu_route_scale_kernel(const T* __restrict__ gu, long gu_
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 const float gg = fminf(gv[j], L), uu = fminf(fmaxf(uv[j], -L), L);
-                gv[j] = w * (gg * sigmoidf_(1.702f * gg) * (uu + 1.f));
+                gv[j] = w * (gg * sigmoidf_(slope * gg) * (uu + 1.f));
             }
         } else {
 #pragma unroll
@@ -489,12 +489,10 @@ int hyb_pool_block_means(const void* k_cache, const void* v_cache, void* k_pool,
                          int prow, int G, int D, int E, int dt, hipStream_t s) {
     if (T_ <= 0) return 0;
     if (pool <= 0 || prow <= 0 || (long)prow * pool < block_size || !slot_mapping) return 1;
-    const int esize = dt == 0 ? 2 : 4;
     const bool vec = D % 4 == 0 && E % 4 == 0 && (size_t)k_cache % 16 == 0 && (size_t)v_cache % 16 == 0;
     const int cv = (D + E) / (vec ? 4 : 1);
     int parts = 256 / cv;
     parts = parts < 1 ? 1 : (parts > pool ? pool : parts);
-    (void)esize;
     const dim3 grid((unsigned)((T_ + POOL_ROWS - 1) / POOL_ROWS), G);
     const size_t lds = (size_t)parts * (D + E) * sizeof(float);
 #define POOL_LAUNCH(VEC)                                                                          \
@@ -581,7 +579,7 @@ int hyb_chosen_route(const void* h, const void* wr, const void* bias, void* dens
 
 int hyb_capped_glu_route_scale(const void* gu, long gu_stride, const void* dense, void* act, long T_,
                                int NE, int NR, int ff, int sff, float limit, float shared_limit,
-                               int dt, hipStream_t s) {
+                               float slope, int dt, hipStream_t s) {
     const int C = NE * ff + sff;
     if (T_ <= 0 || C <= 0) return 0;
     if (!dense || NR < NE) return 1;
@@ -598,7 +596,7 @@ int hyb_capped_glu_route_scale(const void* gu, long gu_stride, const void* dense
                                             dim3(256), 0, s, (const T*)gu + t0 * gu_stride,       \
                                             gu_stride, (const float*)dense + t0 * NR,             \
                                             (T*)act + t0 * (long)C, NE, NR, ff, C, limit,         \
-                                            shared_limit))
+                                            shared_limit, slope))
         if (vec) CGLU(8); else CGLU(1);
 #undef CGLU
     }

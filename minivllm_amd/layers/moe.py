@@ -101,8 +101,10 @@ class CappedRoutedExperts(nn.Module):
     elementwise kernel, no permutation, no host synchronisation."""
 
     def __init__(self, hidden_size: int, ff: int, experts: int, top: int, limit: float,
-                 shared_ff: int = 0, shared_limit: float = 0.0, shared_gate: bool = True):
+                 shared_ff: int = 0, shared_limit: float = 0.0, shared_gate: bool = True,
+                 slope: float = 1.702):
         super().__init__()
+        self.slope = float(slope)
         if not 0 < top <= experts:
             raise ValueError("router: `top` must lie in 1 .. experts")
         self.ff, self.experts, self.top, self.shared_ff = ff, experts, top, shared_ff
@@ -118,5 +120,5 @@ class CappedRoutedExperts(nn.Module):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         route = ops.grouped_route(h, self.router, self.top, 1, 1, "chosen", self.router_bias, self.gates)
         act = ops.capped_glu_route_scale(F.linear(h, self.gate_up), route, self.ff, self.shared_ff,
-                                         self.limit, self.shared_limit, h.dtype)
+                                         self.limit, self.shared_limit, h.dtype, self.slope)
         return F.linear(act, self.down)

@@ -17,8 +17,8 @@ layer of every pass the stream is re-mixed with the embedding output x0: x <- M 
 * feed-forward   ``layers.moe.CappedRoutedExperts``: the router renormalises over the experts it
                  chose, experts clamp their pre-activations, a shared expert with a per-token gate.
 
-The embedding row is scaled on its way into the stream; the output is the final norm and the
-embedding table itself (no scale), times ``logit_scale``.
+The embedding row is scaled on its way into the stream; the head is tied: final norm, then the
+same table (its rows as stored) as the output projection, times ``logit_scale``.
 
 Everything that reads a mixer's normed input is ONE projection (``in_proj`` with one bias
 vector); the stream update and the following norm are one op (``ops.residual_group_norm`` with a
@@ -43,7 +43,7 @@ from minivllm_amd.utils.context import get_context
 
 MIXER_TYPES = ("rglru", "attention")
 RGLRU_SHARPNESS = 8.0           # the constant in the decay's exponent
-EXPERT_SLOPE = 1.702            # g sigmoid(1.702 g): fixed in the experts' activation kernel
+EXPERT_SLOPE = 1.702            # the experts' activation is g sigmoid(1.702 g) (u + 1)
 
 
 # ------------------------------------------------------------------ configuration
@@ -288,7 +288,7 @@ def _make_ff(W: int, f: dict) -> CappedRoutedExperts:
     sh = f.get("shared") or {}
     return CappedRoutedExperts(W, int(f["expert"]["ff"]), int(f["router"]["experts"]),
                                int(f["router"]["top"]), float(f["expert"]["limit"]),
-                               int(sh.get("ff", 0)), float(sh.get("limit", 0.0)))
+                               int(sh.get("ff", 0)), float(sh.get("limit", 0.0)), slope=EXPERT_SLOPE)
 
 
 class ZegelixLayer(nn.Module):

@@ -442,5 +442,6 @@ def rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp
                                  out_dtype)
 
 
-def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype):
-    return _seqmix(gu).capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype)
+def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype, slope=1.702):
+    return _seqmix(gu).capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype,
+                                              slope)

@@ -79,7 +79,7 @@ _utg = _sig("hyb_unturn_gate", _P, _L, _L, _P, _P, _P, _L, _P, _L, _I, _I, _I, _
 _scv = _sig("hyb_short_conv", _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P)
 _lru = _sig("hyb_rglru_scan", _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _F, _I, _I, _P)
 _crt = _sig("hyb_chosen_route", _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P)
-_cgl = _sig("hyb_capped_glu_route_scale", _P, _L, _P, _P, _L, _I, _I, _I, _I, _F, _F, _I, _P)
+_cgl = _sig("hyb_capped_glu_route_scale", _P, _L, _P, _P, _L, _I, _I, _I, _I, _F, _F, _F, _I, _P)
 
 _DT = {torch.bfloat16: 0, torch.float32: 2}
 
@@ -739,7 +739,7 @@ def rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp
     return out
 
 
-def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype):
+def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype, slope=1.702):
     T = gu.shape[0]
     C = gu.shape[1] // 2
     NR = dense.shape[1]
@@ -747,6 +747,6 @@ def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dt
     assert gu.stride(1) == 1 and gu.dtype == out_dtype and C == NE * ff + shared_ff and NR in (NE, NE + 1)
     act = torch.empty((T, C), dtype=out_dtype, device=gu.device)
     _check(_cgl(gu.data_ptr(), _rows(gu), _f32(dense).data_ptr(), act.data_ptr(), T, NE, NR, ff,
-                shared_ff, float(limit), float(shared_limit), _dt(gu), _stream()),
+                shared_ff, float(limit), float(shared_limit), float(slope), _dt(gu), _stream()),
            "capped_glu_route_scale")
     return act

@@ -682,10 +682,10 @@ def rglru_scan(u, gates, gate_bias, lam, y, state, cu_q, positions, slots, sharp
     return (out * gelu_tanh(y.float())).to(out_dtype)
 
 
-def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype):
+def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dtype, slope=1.702):
     """gu [T, 2 C], C = experts * ff + shared_ff: the gate projections of all experts (and of a
     shared one behind them), then their up projections.  Column c: g = min(gate, L), u =
-    clamp(up, -L, L), act = w g sigmoid(1.702 g) (u + 1) with L = ``limit`` for routed columns and
+    clamp(up, -L, L), act = w g sigmoid(slope g) (u + 1) with L = ``limit`` for routed columns and
     ``shared_limit`` for shared ones, w = dense[t, expert] for routed columns (exactly zero where w
     is) and, for shared columns, dense[t, experts] when ``dense`` has that extra column (a
     per-token gate of the shared expert), else 1.  Returns [T, C]."""
@@ -695,7 +695,7 @@ def capped_glu_route_scale(gu, dense, ff, shared_ff, limit, shared_limit, out_dt
     lim = torch.cat([torch.full((ne * ff,), float(limit)), torch.full((shared_ff,), float(shared_limit))])
     g = torch.minimum(g, lim)
     u = torch.maximum(torch.minimum(u, lim), -lim)
-    act = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+    act = g * torch.sigmoid(slope * g) * (u + 1.0)
     sg = dense[:, ne:ne + 1].float() if dense.shape[1] > ne else torch.ones(T, 1)
     w = torch.cat([dense[:, :ne].float().repeat_interleave(ff, 1), sg.expand(T, shared_ff)], 1)
     return torch.where(w != 0, act * w, torch.zeros_like(act)).to(out_dtype)

@@ -204,7 +204,6 @@ def test_conv_and_recurrence_over_steps(dt, C, nb, taps):
             p = to(proj)
             x, y = p[:, :C], p[:, C + 8:]
             state, tail = st[name]
-            kw = dict(row_seq=to(row_seq)) if name == "gpu" else {}
             if name == "gpu":
                 u = mod.short_conv(x, to(w), to(bias), tail, to(cu_q), to(pos), to(seq_slots), to(row_seq))
             else:
